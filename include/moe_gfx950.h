@@ -1,0 +1,141 @@
+/*
+ * C ABI of libmoe_gfx950.so: the fused-MoE expert path for AMD MI355X
+ * (gfx950), a drop-in for the native ops and the Triton grouped GEMM behind
+ * layered-prefill's `nanovllm.ops` / `nanovllm/layers/for_moe/fused_moe.py`.
+ *
+ * Conventions
+ *  - Every pointer is a device pointer on the current HIP device unless its
+ *    name says otherwise.  The library borrows them for the enqueued work
+ *    only; it never allocates, frees or retains device memory, never
+ *    synchronises the device and never copies device -> host.  All launch
+ *    dimensions come from upper bounds known on the host, so each call can be
+ *    recorded into a HIP graph.
+ *  - `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ *  - Return value 0 = enqueued; negative = rejected, nothing enqueued.
+ *    `moe_last_error()` then returns a thread-local, human-readable reason.
+ *  - Scratch memory comes from the caller (`workspace`), sized by the
+ *    matching `*_workspace_bytes` function, 256-byte aligned.
+ */
+#ifndef MOE_GFX950_H_
+#define MOE_GFX950_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* dtype codes for activations / weights / outputs */
+enum MoeDtype { MOE_F32 = 0, MOE_F16 = 1, MOE_BF16 = 2, MOE_E4M3 = 3 };
+/* dtype codes for `topk_ids` handed to moe_align_block_size
+   (csrc/dispatch_utils.h:16-24 dispatches the same integral types) */
+enum MoeIdDtype { MOE_ID_I32 = 0, MOE_ID_I64 = 1, MOE_ID_I16 = 2, MOE_ID_I8 = 3, MOE_ID_U8 = 4 };
+enum MoeActivation { MOE_ACT_SILU = 0, MOE_ACT_SWIGLUOAI = 1, MOE_ACT_GELU = 2 };
+
+enum MoeError {
+  MOE_OK = 0,
+  MOE_ERR_ARG = -1,        /* bad shape / null pointer / unsupported value */
+  MOE_ERR_UNSUPPORTED = -2,/* valid request this build has no kernel for    */
+  MOE_ERR_WORKSPACE = -3,  /* workspace missing or too small                */
+  MOE_ERR_LAUNCH = -4      /* hipLaunchKernel reported an error             */
+};
+
+const char* moe_last_error(void);
+/* ABI version of this header; bumped when a signature changes. */
+int moe_abi_version(void);
+
+/* Replaces `topk_softmax` (csrc/moe_topk_softmax_kernels.cu:476-503, bound at
+ * csrc/ops.cpp:46-51,110-117).  Row-wise fp32 softmax over E experts, then K
+ * rounds of argmax with the lower index winning ties.  Writes
+ * topk_weights[T,K] (softmax values, or those divided by their sum over k when
+ * renormalize != 0, which is nanovllm/layers/for_moe/fused_moe.py:417-418),
+ * topk_ids[T,K] and token_expert_indices[T,K] = k*T + row.  Needs no
+ * workspace for any E in [1, 1024]; requires K <= E. */
+int moe_topk_softmax(const float* gating_output, float* topk_weights, int32_t* topk_ids,
+                     int32_t* token_expert_indices, int T, int E, int K, int renormalize,
+                     void* stream);
+
+/* Replaces `moe_align_block_size` (csrc/moe_align_block_size_kernels.cu:239-291,
+ * bound at csrc/ops.cpp:53-60,119-126).  `sorted_token_ids` (capacity
+ * sorted_cap >= numel + E*(block_size-1)) receives, per expert in ascending
+ * expert order, the flat indices i with topk_ids[i] == e in ascending order,
+ * padded to a multiple of block_size with the value numel; every slot past
+ * the last segment is numel too.  `expert_ids` (capacity expert_cap >=
+ * ceil(sorted_cap/block_size)) names the expert of each block and is 0 past
+ * the last used block.  `num_tokens_post_pad[0]` is the padded total.  Ids
+ * outside [0, E) are dropped.  E <= 1024.  The stable order is produced
+ * without global atomics, so results are deterministic. */
+int64_t moe_align_workspace_bytes(int64_t numel, int E);
+int moe_align_block_size(const void* topk_ids, int ids_dtype, int64_t numel, int E,
+                         int block_size, int32_t* sorted_token_ids, int64_t sorted_cap,
+                         int32_t* expert_ids, int64_t expert_cap, int32_t* num_tokens_post_pad,
+                         void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Replaces `silu_and_mul` (csrc/activation_kernels.cu:68-87, bound at
+ * csrc/ops.cpp:29-31,99-103): out[r,i] = T(silu(in[r,i])) * in[r,d+i]. */
+int moe_silu_and_mul(void* out, const void* in, int64_t rows, int d, int dtype, void* stream);
+
+/* Replaces `swigluoai_and_mul` (csrc/activation_kernels.cu:89-109): gate and
+ * up interleaved along the last dimension. */
+int moe_swigluoai_and_mul(void* out, const void* in, int64_t rows, int d, int dtype, float alpha,
+                          float limit, void* stream);
+
+/* Replaces `moe_sum` (nanovllm/layers/for_moe/moe_easy_kernel.py:26-31):
+ * out[t,:] = sum_k in[t,k,:], fp32 accumulation, one rounding. */
+int moe_sum(void* out, const void* in, int64_t T, int K, int H, int dtype, void* stream);
+
+/* Replaces the body of `fused_experts_impl` after alignment
+ * (nanovllm/layers/for_moe/fused_moe.py:579-631): grouped GEMM x*W13^T with the
+ * gated activation fused into its epilogue, grouped GEMM with W2^T times the
+ * routed weight, and the top-k combine.  `out` may alias `x` (inplace=True at
+ * nanovllm/layers/fused_moe.py:203-216). */
+typedef struct MoeFusedExpertsArgs {
+  /* tensors */
+  const void* x;             /* [T, H] activations, row-major contiguous            */
+  void* out;                 /* [T, H] result, same dtype as x                      */
+  const void* w13;           /* [E, 2I, H] gate rows [0,I) then up rows [I,2I)      */
+  const void* w2;            /* [E, H, I]                                           */
+  const void* w13_bias;      /* [E, 2I] or NULL                                     */
+  const void* w2_bias;       /* [E, H] or NULL                                      */
+  const float* w13_scale;    /* fp8 only: [E, 2I] per-output-channel scales, else NULL */
+  const float* w2_scale;     /* fp8 only: [E, H], else NULL                         */
+  const float* topk_weights; /* [T, K] fp32                                          */
+  const int32_t* sorted_token_ids;    /* from moe_align_block_size                  */
+  const int32_t* expert_ids;
+  const int32_t* num_tokens_post_pad; /* read on the device only                    */
+  void* workspace;
+  int64_t workspace_bytes;
+  /* element strides of the expert dimension and the row dimension of the
+     weights (last dimension is contiguous) */
+  int64_t w13_stride_e, w13_stride_n, w2_stride_e, w2_stride_n;
+  /* sizes */
+  int32_t T, H, I, E, K;
+  int32_t block_size;        /* the block_size the alignment was made with          */
+  int64_t sorted_cap;        /* numel + E*(block_size-1)                             */
+  int32_t act_dtype;         /* MoeDtype of x / out / biases                         */
+  int32_t weight_dtype;      /* MoeDtype of w13 / w2 (MOE_E4M3 selects the fp8 path) */
+  int32_t activation;        /* MoeActivation                                        */
+  int32_t apply_router_weight_on_input;
+  float swiglu_alpha, swiglu_limit;
+  void* stream;
+} MoeFusedExpertsArgs;
+
+int64_t moe_fused_experts_workspace_bytes(int T, int H, int I, int E, int K, int block_size,
+                                          int act_dtype, int weight_dtype);
+int moe_fused_experts(const MoeFusedExpertsArgs* args);
+
+/* The M-tile (alignment block_size) the grouped GEMMs run best with for M
+ * tokens; plays the role of config["BLOCK_SIZE_M"] chosen by
+ * try_get_optimal_moe_config (nanovllm/layers/for_moe/fused_moe.py:354-390). */
+int moe_preferred_block_size(int M, int E, int K, int act_dtype, int weight_dtype);
+
+/* fp8 helpers (no counterpart in the reference, which asserts the scales are
+ * None at nanovllm/layers/for_moe/fused_moe.py:248-249): per-output-channel
+ * e4m3 quantisation of a [rows, cols] weight matrix, s[r] = amax|w[r,:]|/448. */
+int moe_quant_rows_e4m3(const void* w, int src_dtype, int64_t rows, int cols, uint8_t* q,
+                        float* scales, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOE_GFX950_H_ */

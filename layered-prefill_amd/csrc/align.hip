@@ -1,0 +1,312 @@
+// Expert-sorted token alignment (counting sort by expert, padded to blocks).
+//
+// Replaces moe_align_block_size_kernel + count_and_sort_expert_tokens_kernel of
+// the reference (csrc/moe_align_block_size_kernels.cu:140-237).  The reference
+// ranks tokens inside an expert's segment with a global atomicAdd, which makes
+// the order arbitrary; here the flat index range is cut into contiguous
+// segments, one wavefront per segment, and a token's rank is
+//     (tokens of its expert in earlier segments)            -- prefix over segments
+//   + (tokens of its expert earlier in this segment)        -- running LDS counter
+//   + (same-expert lanes below it in the current 64 ids)    -- ballot + popcount
+// which is the stable order and needs no global atomics.
+//
+// Small inputs run as ONE workgroup of 16 wavefronts (histogram, scans and
+// scatter in LDS); larger ones as three launches (count / scan / scatter)
+// with the per-segment histograms in the caller's workspace.
+#include "common.h"
+
+namespace {
+
+constexpr int kMaxExperts = 1024;
+constexpr int kScanThreads = 1024;              // one thread per expert in the scans
+constexpr int kScanWaves = kScanThreads / kWave;
+constexpr int kSegLen = 512;                    // ids per wavefront segment, large path
+constexpr int64_t kSmallNumel = 16384;          // at or below: single-workgroup path ...
+constexpr int kSmallMaxExperts = 512;           // ... when its LDS histograms fit in 64 KB
+
+__device__ __forceinline__ int load_id(const void* ids, int dtype, int64_t i) {
+  switch (dtype) {
+    case MOE_ID_I32: return static_cast<const int32_t*>(ids)[i];
+    case MOE_ID_I64: {
+      int64_t v = static_cast<const int64_t*>(ids)[i];
+      return (v < 0 || v > INT32_MAX) ? -1 : static_cast<int>(v);
+    }
+    case MOE_ID_I16: return static_cast<const int16_t*>(ids)[i];
+    case MOE_ID_I8: return static_cast<const int8_t*>(ids)[i];
+    default: return static_cast<const uint8_t*>(ids)[i];
+  }
+}
+
+// Lanes of the wavefront whose (valid) id equals this lane's id.
+__device__ __forceinline__ uint64_t same_id_lanes(int id, bool valid, int id_bits) {
+  uint64_t m = __ballot(valid);
+  for (int b = 0; b < id_bits; ++b) {
+    const bool bit = (id >> b) & 1;
+    const uint64_t bal = __ballot(bit);
+    m &= bit ? bal : ~bal;
+  }
+  return m;
+}
+
+__device__ __forceinline__ uint64_t lanes_below(int lane) { return (1ull << lane) - 1ull; }
+
+// Exclusive prefix sum of one int per thread over a kScanThreads workgroup.
+// `wave_tot` is LDS scratch of kScanWaves + 1 ints; slot kScanWaves receives
+// the grand total.  Contains workgroup barriers.
+__device__ int block_exclusive_scan(int v, volatile int* wave_tot) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  int inc = v;
+#pragma unroll
+  for (int d = 1; d < kWave; d *= 2) {
+    int o = __shfl_up(inc, d, kWave);
+    if (lane >= d) inc += o;
+  }
+  if (lane == kWave - 1) wave_tot[wave] = inc;
+  __syncthreads();
+  if (wave == 0) {
+    int w = lane < kScanWaves ? wave_tot[lane] : 0;
+    int winc = w;
+#pragma unroll
+    for (int d = 1; d < kScanWaves; d *= 2) {
+      int o = __shfl_up(winc, d, kWave);
+      if (lane >= d) winc += o;
+    }
+    if (lane < kScanWaves) wave_tot[lane] = winc - w;
+    if (lane == kScanWaves - 1) wave_tot[kScanWaves] = winc;
+  }
+  __syncthreads();
+  return inc - v + wave_tot[wave];
+}
+
+// After `cum[0..E]` (LDS) holds the padded exclusive prefix and `tot[e]` the
+// raw counts: writes expert_ids, num_tokens_post_pad and every padding slot
+// of sorted_token_ids.  Called by all kScanThreads threads.
+__device__ void write_blocks_and_padding(const volatile int* cum, const volatile int* tot, int E,
+                                         int BM, int numel, int32_t* sorted_ids,
+                                         int64_t sorted_cap, int32_t* expert_ids,
+                                         int64_t expert_cap, int32_t* num_post_pad) {
+  const int total = cum[E];
+  if (threadIdx.x == 0) *num_post_pad = total;
+  const int used_blocks = total / BM;
+  for (int b = threadIdx.x; b < used_blocks; b += kScanThreads) {
+    const int pos = b * BM;
+    // first j in [1, E] with cum[j] > pos; the block belongs to expert j - 1
+    int lo = 1, hi = E;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (cum[mid] > pos) hi = mid; else lo = mid + 1;
+    }
+    expert_ids[b] = lo - 1;
+  }
+  for (int64_t b = used_blocks + threadIdx.x; b < expert_cap; b += kScanThreads) expert_ids[b] = 0;
+  // padding inside each expert's last block: one wavefront per expert
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  for (int e = wave; e < E; e += kScanWaves) {
+    const int beg = cum[e] + tot[e], end = cum[e + 1];
+    for (int p = beg + lane; p < end; p += kWave) sorted_ids[p] = numel;
+  }
+  for (int64_t p = total + threadIdx.x; p < sorted_cap; p += kScanThreads) sorted_ids[p] = numel;
+}
+
+// Walks ids [beg, end) in order, 64 at a time, and writes each flat index to
+// its slot.  `run[e]` (LDS, private to this wavefront) holds the next free
+// slot of expert e and is advanced by the lowest lane of every same-id group.
+__device__ __forceinline__ void scatter_segment(const void* ids, int dtype, int64_t beg,
+                                                int64_t end, int E, int id_bits,
+                                                volatile int* run, int32_t* sorted_ids) {
+  const int lane = threadIdx.x % kWave;
+  for (int64_t base = beg; base < end; base += kWave) {
+    const int64_t i = base + lane;
+    int id = -1;
+    if (i < end) id = load_id(ids, dtype, i);
+    const bool valid = id >= 0 && id < E;
+    const uint64_t grp = same_id_lanes(id, valid, id_bits);
+    if (valid) {
+      const int below = __popcll(grp & lanes_below(lane));
+      const int slot = run[id] + below;
+      sorted_ids[slot] = static_cast<int32_t>(i);
+      if (below == 0) run[id] = slot + __popcll(grp);
+    }
+  }
+}
+
+__global__ __launch_bounds__(kScanThreads) void align_small_kernel(
+    const void* __restrict__ ids, int dtype, int numel, int E, int BM, int id_bits,
+    int32_t* __restrict__ sorted_ids, int64_t sorted_cap, int32_t* __restrict__ expert_ids,
+    int64_t expert_cap, int32_t* __restrict__ num_post_pad) {
+  extern __shared__ int lds[];
+  // layout: seg_cnt[kScanWaves][E] | cum[E+1] | tot[E] | wave_tot[kScanWaves+1]
+  volatile int* seg_cnt = lds;
+  volatile int* cum = lds + kScanWaves * E;
+  volatile int* tot = cum + (E + 1);
+  volatile int* wave_tot = tot + E;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int seg_len = ((numel + kScanWaves - 1) / kScanWaves + kWave - 1) / kWave * kWave;
+  const int beg = min(wave * seg_len, numel), end = min(beg + seg_len, numel);
+
+  for (int i = threadIdx.x; i < kScanWaves * E; i += kScanThreads) seg_cnt[i] = 0;
+  __syncthreads();
+  for (int i = beg + lane; i < end; i += kWave) {
+    const int id = load_id(ids, dtype, i);
+    if (id >= 0 && id < E) atomicAdd(const_cast<int*>(&seg_cnt[wave * E + id]), 1);
+  }
+  __syncthreads();
+  int padded = 0;
+  if (threadIdx.x < E) {
+    const int e = threadIdx.x;
+    int running = 0;
+    for (int w = 0; w < kScanWaves; ++w) {
+      const int c = seg_cnt[w * E + e];
+      seg_cnt[w * E + e] = running;
+      running += c;
+    }
+    tot[e] = running;
+    padded = (running + BM - 1) / BM * BM;
+  }
+  const int excl = block_exclusive_scan(padded, wave_tot);
+  if (threadIdx.x < E) cum[threadIdx.x] = excl;
+  if (threadIdx.x == E) cum[E] = excl;  // E < kScanThreads: threads past E add 0
+  if (E == kScanThreads && threadIdx.x == 0) cum[E] = wave_tot[kScanWaves];
+  __syncthreads();
+  write_blocks_and_padding(cum, tot, E, BM, numel, sorted_ids, sorted_cap, expert_ids, expert_cap,
+                           num_post_pad);
+  // per-wavefront running slots: segment prefix + expert base
+  for (int e = lane; e < E; e += kWave) seg_cnt[wave * E + e] += cum[e];
+  scatter_segment(ids, dtype, beg, end, E, id_bits, seg_cnt + wave * E, sorted_ids);
+}
+
+// ---- large path -----------------------------------------------------------
+__global__ __launch_bounds__(kWave) void align_count_kernel(const void* __restrict__ ids, int dtype,
+                                                            int64_t numel, int E,
+                                                            int32_t* __restrict__ seg_cnt) {
+  extern __shared__ int lds[];
+  const int lane = threadIdx.x;
+  for (int e = lane; e < E; e += kWave) lds[e] = 0;
+  __syncthreads();
+  const int64_t beg = static_cast<int64_t>(blockIdx.x) * kSegLen;
+  const int64_t end = beg + kSegLen < numel ? beg + kSegLen : numel;
+  for (int64_t i = beg + lane; i < end; i += kWave) {
+    const int id = load_id(ids, dtype, i);
+    if (id >= 0 && id < E) atomicAdd(&lds[id], 1);
+  }
+  __syncthreads();
+  for (int e = lane; e < E; e += kWave) seg_cnt[static_cast<size_t>(blockIdx.x) * E + e] = lds[e];
+}
+
+__global__ __launch_bounds__(kScanThreads) void align_scan_kernel(
+    int32_t* __restrict__ seg_cnt, int nseg, int E, int BM, int numel,
+    int32_t* __restrict__ cum_out, int32_t* __restrict__ sorted_ids, int64_t sorted_cap,
+    int32_t* __restrict__ expert_ids, int64_t expert_cap, int32_t* __restrict__ num_post_pad) {
+  __shared__ int s_cum[kMaxExperts + 1];
+  __shared__ int s_tot[kMaxExperts];
+  __shared__ int s_wave_tot[kScanWaves + 1];
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  // per expert: exclusive prefix of its counts over segments (in place)
+  for (int e = wave; e < E; e += kScanWaves) {
+    int running = 0;
+    for (int s0 = 0; s0 < nseg; s0 += kWave) {
+      const int s = s0 + lane;
+      const int c = s < nseg ? seg_cnt[static_cast<size_t>(s) * E + e] : 0;
+      int inc = c;
+#pragma unroll
+      for (int d = 1; d < kWave; d *= 2) {
+        int o = __shfl_up(inc, d, kWave);
+        if (lane >= d) inc += o;
+      }
+      if (s < nseg) seg_cnt[static_cast<size_t>(s) * E + e] = running + inc - c;
+      running += __shfl(inc, kWave - 1, kWave);
+    }
+    if (lane == 0) s_tot[e] = running;
+  }
+  __syncthreads();
+  int padded = 0;
+  if (threadIdx.x < E) padded = (s_tot[threadIdx.x] + BM - 1) / BM * BM;
+  const int excl = block_exclusive_scan(padded, s_wave_tot);
+  if (threadIdx.x < E) s_cum[threadIdx.x] = excl;
+  if (threadIdx.x == E) s_cum[E] = excl;
+  if (E == kScanThreads && threadIdx.x == 0) s_cum[E] = s_wave_tot[kScanWaves];
+  __syncthreads();
+  for (int e = threadIdx.x; e <= E; e += kScanThreads) cum_out[e] = s_cum[e];
+  write_blocks_and_padding(s_cum, s_tot, E, BM, numel, sorted_ids, sorted_cap, expert_ids,
+                           expert_cap, num_post_pad);
+}
+
+__global__ __launch_bounds__(kWave) void align_scatter_kernel(
+    const void* __restrict__ ids, int dtype, int64_t numel, int E, int id_bits,
+    const int32_t* __restrict__ seg_base, const int32_t* __restrict__ cum,
+    int32_t* __restrict__ sorted_ids) {
+  extern __shared__ int lds[];
+  const int lane = threadIdx.x;
+  for (int e = lane; e < E; e += kWave)
+    lds[e] = seg_base[static_cast<size_t>(blockIdx.x) * E + e] + cum[e];
+  __syncthreads();
+  const int64_t beg = static_cast<int64_t>(blockIdx.x) * kSegLen;
+  const int64_t end = beg + kSegLen < numel ? beg + kSegLen : numel;
+  scatter_segment(ids, dtype, beg, end, E, id_bits, lds, sorted_ids);
+}
+
+int bits_for(int E) {
+  int b = 1;
+  while ((1 << b) < E) ++b;
+  return b;
+}
+
+}  // namespace
+
+MOE_EXPORT int64_t moe_align_workspace_bytes(int64_t numel, int E) {
+  if (numel < 0 || E < 1) return 0;
+  if (numel <= kSmallNumel && E <= kSmallMaxExperts) return 0;
+  const int64_t nseg = numel > 0 ? (numel + kSegLen - 1) / kSegLen : 1;
+  return moe_align_up((nseg * E + E + 1) * static_cast<int64_t>(sizeof(int32_t)), 256);
+}
+
+MOE_EXPORT int moe_align_block_size(const void* topk_ids, int ids_dtype, int64_t numel, int E,
+                                    int block_size, int32_t* sorted_token_ids, int64_t sorted_cap,
+                                    int32_t* expert_ids, int64_t expert_cap,
+                                    int32_t* num_tokens_post_pad, void* workspace,
+                                    int64_t workspace_bytes, void* stream) {
+  if (numel < 0 || E < 1 || block_size < 1)
+    return moe_fail(MOE_ERR_ARG, "moe_align_block_size: bad sizes numel=%lld E=%d block_size=%d",
+                    static_cast<long long>(numel), E, block_size);
+  if (E > kMaxExperts)
+    return moe_fail(MOE_ERR_UNSUPPORTED, "moe_align_block_size: num_experts %d > %d", E, kMaxExperts);
+  if (ids_dtype < MOE_ID_I32 || ids_dtype > MOE_ID_U8)
+    return moe_fail(MOE_ERR_ARG, "moe_align_block_size: unknown id dtype code %d", ids_dtype);
+  const int64_t need_sorted = numel + static_cast<int64_t>(E) * (block_size - 1);
+  if (need_sorted > INT32_MAX)
+    return moe_fail(MOE_ERR_ARG, "moe_align_block_size: padded length overflows int32");
+  if (sorted_cap < need_sorted)
+    return moe_fail(MOE_ERR_ARG, "moe_align_block_size: sorted_token_ids holds %lld, needs %lld",
+                    static_cast<long long>(sorted_cap), static_cast<long long>(need_sorted));
+  if (expert_cap < (need_sorted + block_size - 1) / block_size)
+    return moe_fail(MOE_ERR_ARG, "moe_align_block_size: expert_ids holds %lld, needs %lld",
+                    static_cast<long long>(expert_cap),
+                    static_cast<long long>((need_sorted + block_size - 1) / block_size));
+  if (!sorted_token_ids || !expert_ids || !num_tokens_post_pad || (numel > 0 && !topk_ids))
+    return moe_fail(MOE_ERR_ARG, "moe_align_block_size: null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int id_bits = bits_for(E);
+  if (numel <= kSmallNumel && E <= kSmallMaxExperts) {
+    const size_t lds = (static_cast<size_t>(kScanWaves) * E + (E + 1) + E + kScanWaves + 1) * sizeof(int);
+    hipLaunchKernelGGL(align_small_kernel, dim3(1), dim3(kScanThreads), lds, s, topk_ids, ids_dtype,
+                       static_cast<int>(numel), E, block_size, id_bits, sorted_token_ids,
+                       sorted_cap, expert_ids, expert_cap, num_tokens_post_pad);
+    return moe_check_launch("moe_align_block_size (single workgroup)");
+  }
+  const int64_t need_ws = moe_align_workspace_bytes(numel, E);
+  if (!workspace || workspace_bytes < need_ws)
+    return moe_fail(MOE_ERR_WORKSPACE, "moe_align_block_size: workspace %lld B, needs %lld B",
+                    static_cast<long long>(workspace_bytes), static_cast<long long>(need_ws));
+  const int nseg = numel > 0 ? static_cast<int>((numel + kSegLen - 1) / kSegLen) : 1;
+  int32_t* seg_cnt = static_cast<int32_t*>(workspace);
+  int32_t* cum = seg_cnt + static_cast<size_t>(nseg) * E;
+  hipLaunchKernelGGL(align_count_kernel, dim3(nseg), dim3(kWave), E * sizeof(int), s, topk_ids,
+                     ids_dtype, numel, E, seg_cnt);
+  hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, seg_cnt, nseg, E,
+                     block_size, static_cast<int>(numel), cum, sorted_token_ids, sorted_cap,
+                     expert_ids, expert_cap, num_tokens_post_pad);
+  hipLaunchKernelGGL(align_scatter_kernel, dim3(nseg), dim3(kWave), E * sizeof(int), s, topk_ids,
+                     ids_dtype, numel, E, id_bits, seg_cnt, cum,
+                     sorted_token_ids);
+  return moe_check_launch("moe_align_block_size");
+}

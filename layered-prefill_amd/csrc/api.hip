@@ -1,0 +1,27 @@
+// Error reporting shared by every entry point of libmoe_gfx950.so.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "common.h"
+
+namespace {
+thread_local char g_last_error[512] = "";
+}
+
+int moe_fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int moe_check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return MOE_OK;
+  return moe_fail(MOE_ERR_LAUNCH, "%s: kernel launch failed: %s", what, hipGetErrorString(e));
+}
+
+MOE_EXPORT const char* moe_last_error(void) { return g_last_error; }
+
+MOE_EXPORT int moe_abi_version(void) { return 1; }

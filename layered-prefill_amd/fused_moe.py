@@ -1,0 +1,207 @@
+"""Host side of the fused-MoE expert path, mirroring the reference's
+``nanovllm/layers/for_moe/fused_moe.py`` (same function names, argument order,
+defaults, assertions and return values) on top of libmoe_gfx950.so.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib, ops
+from ._lib import MoeFusedExpertsArgs, check, lib, stream_ptr
+
+
+def cdiv(a: int, b: int) -> int:
+    return -(-a // b)
+
+
+def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: int
+                         ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """nanovllm/layers/for_moe/fused_moe.py:17-70.  Returns (sorted_token_ids
+    [numel + E*(block_size-1)], expert_ids [ceil(that / block_size)],
+    num_tokens_post_padded [1]), all int32 on topk_ids' device.  The kernel
+    writes every element of all three, so nothing is pre-filled here."""
+    max_num_tokens_padded = topk_ids.numel() + num_experts * (block_size - 1)
+    sorted_ids = torch.empty((max_num_tokens_padded,), dtype=torch.int32, device=topk_ids.device)
+    max_num_m_blocks = cdiv(max_num_tokens_padded, block_size)
+    expert_ids = torch.empty((max_num_m_blocks,), dtype=torch.int32, device=topk_ids.device)
+    num_tokens_post_pad = torch.empty((1), dtype=torch.int32, device=topk_ids.device)
+    ops.moe_align_block_size(topk_ids, num_experts, block_size, sorted_ids, expert_ids,
+                             num_tokens_post_pad)
+    return sorted_ids, expert_ids, num_tokens_post_pad
+
+
+def try_get_optimal_moe_config(w1_shape, w2_shape, top_k: int, dtype: Optional[str], M: int,
+                               is_marlin: bool = False,
+                               block_shape: Optional[list] = None) -> dict:
+    """Role of nanovllm/layers/for_moe/fused_moe.py:354-390.  The reference looks
+    up Triton tile tables per device name; the HIP kernels own their tiling, so
+    the only entry that still matters to callers is BLOCK_SIZE_M, the block size
+    handed to moe_align_block_size."""
+    E = w2_shape[0]
+    bm = lib().moe_preferred_block_size(M, E, top_k, _lib.DTYPE_CODE[torch.bfloat16],
+                                        _lib.DTYPE_CODE[torch.bfloat16])
+    return {"BLOCK_SIZE_M": bm}
+
+
+def fused_topk(hidden_states: torch.Tensor, gating_output: torch.Tensor, topk: int,
+               renormalize: bool):
+    """nanovllm/layers/for_moe/fused_moe.py:393-419."""
+    assert hidden_states.shape[0] == gating_output.shape[0], "Number of tokens mismatch"
+    M, _ = hidden_states.shape
+    topk_weights = torch.empty(M, topk, dtype=torch.float32, device=hidden_states.device)
+    topk_ids = torch.empty(M, topk, dtype=torch.int32, device=hidden_states.device)
+    token_expert_indicies = torch.empty(M, topk, dtype=torch.int32, device=hidden_states.device)
+    gating = gating_output if gating_output.dtype == torch.float32 else gating_output.float()
+    ops.topk_softmax(topk_weights, topk_ids, token_expert_indicies, gating.contiguous(),
+                     renormalize=renormalize)
+    return topk_weights, topk_ids, token_expert_indicies
+
+
+def fused_experts(hidden_states: torch.Tensor,
+                  w1: torch.Tensor,
+                  w2: torch.Tensor,
+                  w1_bias: Optional[torch.Tensor],
+                  w2_bias: Optional[torch.Tensor],
+                  topk_weights: torch.Tensor,
+                  topk_ids: torch.Tensor,
+                  inplace: bool = False,
+                  activation: str = "silu",
+                  apply_router_weight_on_input: bool = False,
+                  per_channel_quant: bool = False,
+                  global_num_experts: int = -1,
+                  expert_map: Optional[torch.Tensor] = None,
+                  w1_scale: Optional[torch.Tensor] = None,
+                  w2_scale: Optional[torch.Tensor] = None,
+                  w1_zp: Optional[torch.Tensor] = None,
+                  w2_zp: Optional[torch.Tensor] = None,
+                  a1_scale: Optional[torch.Tensor] = None,
+                  a2_scale: Optional[torch.Tensor] = None,
+                  block_shape: Optional[list] = None,
+                  allow_deep_gemm: bool = False) -> torch.Tensor:
+    """nanovllm/layers/for_moe/fused_moe.py:422-460."""
+    if inplace:
+        fused_experts_impl(hidden_states, w1, w2, topk_weights, topk_ids, True, activation,
+                           apply_router_weight_on_input, per_channel_quant, global_num_experts,
+                           expert_map, w1_scale, w2_scale, w1_zp, w2_zp, a1_scale, a2_scale,
+                           block_shape, w1_bias, w2_bias)
+        return hidden_states
+    return fused_experts_impl(hidden_states, w1, w2, topk_weights, topk_ids, False, activation,
+                              apply_router_weight_on_input, per_channel_quant, global_num_experts,
+                              expert_map, w1_scale, w2_scale, w1_zp, w2_zp, a1_scale, a2_scale,
+                              block_shape, w1_bias, w2_bias)
+
+
+_FP8_DTYPES = tuple(getattr(torch, n) for n in ("float8_e4m3fn",) if hasattr(torch, n))
+
+
+def fused_experts_impl(hidden_states: torch.Tensor,
+                       w1: torch.Tensor,
+                       w2: torch.Tensor,
+                       topk_weights: torch.Tensor,
+                       topk_ids: torch.Tensor,
+                       inplace: bool = False,
+                       activation: str = "silu",
+                       apply_router_weight_on_input: bool = False,
+                       per_channel_quant: bool = False,
+                       global_num_experts: int = -1,
+                       expert_map: Optional[torch.Tensor] = None,
+                       w1_scale: Optional[torch.Tensor] = None,
+                       w2_scale: Optional[torch.Tensor] = None,
+                       w1_zp: Optional[torch.Tensor] = None,
+                       w2_zp: Optional[torch.Tensor] = None,
+                       a1_scale: Optional[torch.Tensor] = None,
+                       a2_scale: Optional[torch.Tensor] = None,
+                       block_shape: Optional[list] = None,
+                       w1_bias: Optional[torch.Tensor] = None,
+                       w2_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """nanovllm/layers/for_moe/fused_moe.py:461-633: align -> gate-up GEMM with
+    the gated activation -> down GEMM times the routed weight -> top-k sum, in
+    chunks of 64K tokens."""
+    # Check constraints (same wording as the reference, :484-493).
+    assert hidden_states.size(1) == w1.size(2), (
+        f"Hidden size mismatch {hidden_states.size(1)} != {w1.size(2)}")
+    assert topk_weights.size() == topk_ids.size(), "topk shape mismatch"
+    assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
+    assert w1.stride(-1) == 1, "Stride of last dimension must be 1"
+    assert w2.stride(-1) == 1, "Stride of last dimension must be 1"
+    assert hidden_states.dtype in [torch.float32, torch.float16, torch.bfloat16]
+    assert a1_scale is None and a2_scale is None, \
+        "static activation scales are not supported (fp8 activations are quantised per token)"
+    assert w1_zp is None and w2_zp is None and block_shape is None and expert_map is None
+    if activation not in _lib.ACTIVATION_CODE:
+        raise ValueError(f"Unsupported FusedMoe activation: {activation}")
+    _lib.require_gpu_tensor(hidden_states, "hidden_states")
+
+    fp8 = w1.dtype in _FP8_DTYPES or (w1_scale is not None)
+    if fp8:
+        assert w1_scale is not None and w2_scale is not None, "fp8 weights need w1_scale and w2_scale"
+        weight_code = _lib.E4M3_CODE
+    else:
+        assert w1.dtype == hidden_states.dtype and w2.dtype == hidden_states.dtype, \
+            "weights and activations must share a dtype"
+        weight_code = _lib.DTYPE_CODE[w1.dtype]
+
+    num_tokens = hidden_states.size(0)
+    E, N, _ = w1.size()
+    K = w2.size(1)
+    assert w2.size(2) == N // 2 and w2.size(0) == E, "w2 must be [E, H, I] for w1 [E, 2I, H]"
+    if global_num_experts == -1:
+        global_num_experts = E
+    top_k_num = topk_ids.size(1)
+    CHUNK_SIZE: int = 64 * 1024
+    M = min(num_tokens, CHUNK_SIZE)
+    config = try_get_optimal_moe_config(w1.size(), w2.size(), top_k_num, None, M)
+
+    out_hidden_states = hidden_states if inplace else torch.empty_like(hidden_states)
+    if topk_weights.dtype != torch.float32:
+        topk_weights = topk_weights.float()
+    if topk_ids.dtype != torch.int32:
+        topk_ids = topk_ids.to(torch.int32)
+    topk_weights = topk_weights.contiguous()
+    topk_ids = topk_ids.contiguous()
+
+    L = lib()
+    dev = hidden_states.device
+    act_code = _lib.DTYPE_CODE[hidden_states.dtype]
+    for chunk in range((num_tokens // CHUNK_SIZE) + 1):
+        begin, end = chunk * CHUNK_SIZE, min((chunk + 1) * CHUNK_SIZE, num_tokens)
+        tokens_in_chunk = end - begin
+        if tokens_in_chunk <= 0:
+            break
+        if tokens_in_chunk < CHUNK_SIZE and chunk > 0:
+            config = try_get_optimal_moe_config(w1.size(), w2.size(), top_k_num, None,
+                                                tokens_in_chunk)
+        bm = config["BLOCK_SIZE_M"]
+        curr_ids = topk_ids[begin:end]
+        curr_w = topk_weights[begin:end]
+        sorted_token_ids, expert_ids, num_tokens_post_padded = moe_align_block_size(
+            curr_ids, bm, global_num_experts)
+        ws_bytes = L.moe_fused_experts_workspace_bytes(tokens_in_chunk, K, N // 2, E, top_k_num, bm,
+                                                       act_code, weight_code)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        args = MoeFusedExpertsArgs(
+            x=hidden_states[begin:end].data_ptr(), out=out_hidden_states[begin:end].data_ptr(),
+            w13=w1.data_ptr(), w2=w2.data_ptr(),
+            w13_bias=w1_bias.data_ptr() if w1_bias is not None else None,
+            w2_bias=w2_bias.data_ptr() if w2_bias is not None else None,
+            w13_scale=w1_scale.data_ptr() if w1_scale is not None else None,
+            w2_scale=w2_scale.data_ptr() if w2_scale is not None else None,
+            topk_weights=curr_w.data_ptr(), sorted_token_ids=sorted_token_ids.data_ptr(),
+            expert_ids=expert_ids.data_ptr(), num_tokens_post_pad=num_tokens_post_padded.data_ptr(),
+            workspace=workspace.data_ptr(), workspace_bytes=ws_bytes,
+            w13_stride_e=w1.stride(0), w13_stride_n=w1.stride(1),
+            w2_stride_e=w2.stride(0), w2_stride_n=w2.stride(1),
+            T=tokens_in_chunk, H=K, I=N // 2, E=E, K=top_k_num, block_size=bm,
+            sorted_cap=sorted_token_ids.numel(), act_dtype=act_code, weight_dtype=weight_code,
+            activation=_lib.ACTIVATION_CODE[activation],
+            apply_router_weight_on_input=int(apply_router_weight_on_input),
+            swiglu_alpha=1.702, swiglu_limit=7.0, stream=stream_ptr(dev))
+        if w1_bias is not None:
+            assert w1_bias.is_contiguous() and w1_bias.dtype == hidden_states.dtype
+        if w2_bias is not None:
+            assert w2_bias.is_contiguous() and w2_bias.dtype == hidden_states.dtype
+        with torch.cuda.device(dev):
+            check(L.moe_fused_experts(args))
+    return out_hidden_states

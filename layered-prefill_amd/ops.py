@@ -1,0 +1,148 @@
+"""Native ops with the signatures of the reference's ``nanovllm.ops`` module
+(pybind bindings at csrc/ops.cpp:29-60,97-133 of the reference): out-parameter
+style, nothing returned, work enqueued on torch's current stream.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from ._lib import check, lib, require_gpu_tensor, stream_ptr
+
+# scratch for the three-launch alignment path, one buffer per (device, stream)
+# so that concurrent streams never share it; grown on demand, never shrunk
+_align_ws: dict = {}
+
+
+def _align_workspace(nbytes: int, device: torch.device) -> torch.Tensor:
+    key = (device.index, stream_ptr(device))
+    buf = _align_ws.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 16), dtype=torch.uint8, device=device)
+        _align_ws[key] = buf
+    return buf
+
+
+def topk_softmax(topk_weights: torch.Tensor, topk_indices: torch.Tensor,
+                 token_expert_indices: torch.Tensor, gating_output: torch.Tensor,
+                 renormalize: bool = False) -> None:
+    """csrc/moe_topk_softmax_kernels.cu:476-503.  ``renormalize`` (not in the
+    reference op; default off) folds nanovllm/layers/for_moe/fused_moe.py:417-418
+    into the same launch."""
+    require_gpu_tensor(gating_output, "gating_output")
+    if gating_output.dtype != torch.float32:
+        raise RuntimeError(f"expected scalar type Float but found {gating_output.dtype}")
+    if topk_weights.dtype != torch.float32:
+        raise RuntimeError(f"expected scalar type Float but found {topk_weights.dtype}")
+    if topk_indices.dtype != torch.int32 or token_expert_indices.dtype != torch.int32:
+        raise RuntimeError("expected scalar type Int for topk_indices / token_expert_indices")
+    for name, t in (("topk_weights", topk_weights), ("topk_indices", topk_indices),
+                    ("token_expert_indices", token_expert_indices),
+                    ("gating_output", gating_output)):
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous")
+    E = gating_output.size(-1)
+    T = gating_output.numel() // E if E else 0
+    K = topk_weights.size(-1)
+    if topk_weights.numel() != T * K or topk_indices.numel() != T * K \
+            or token_expert_indices.numel() != T * K:
+        raise RuntimeError("topk_softmax: output tensors must hold num_tokens * topk elements")
+    with torch.cuda.device(gating_output.device):
+        check(lib().moe_topk_softmax(gating_output.data_ptr(), topk_weights.data_ptr(),
+                                     topk_indices.data_ptr(), token_expert_indices.data_ptr(),
+                                     T, E, K, int(renormalize), stream_ptr(gating_output.device)))
+
+
+def moe_align_block_size(topk_ids: torch.Tensor, num_experts: int, block_size: int,
+                         sorted_token_ids: torch.Tensor, experts_ids: torch.Tensor,
+                         num_tokens_post_pad: torch.Tensor) -> None:
+    """csrc/moe_align_block_size_kernels.cu:239-291."""
+    require_gpu_tensor(topk_ids, "topk_ids")
+    if topk_ids.dtype not in _lib.ID_DTYPE_CODE:
+        raise RuntimeError(f"moe_align_block_size_kernel not implemented for '{topk_ids.dtype}'")
+    for name, t in (("sorted_token_ids", sorted_token_ids), ("experts_ids", experts_ids),
+                    ("num_tokens_post_pad", num_tokens_post_pad)):
+        if t.dtype != torch.int32:
+            raise RuntimeError(f"expected scalar type Int but found {t.dtype} for {name}")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous")
+    if not topk_ids.is_contiguous():
+        raise RuntimeError("topk_ids must be contiguous")
+    numel = topk_ids.numel()
+    L = lib()
+    ws_bytes = L.moe_align_workspace_bytes(numel, num_experts)
+    ws = _align_workspace(ws_bytes, topk_ids.device) if ws_bytes else None
+    with torch.cuda.device(topk_ids.device):
+        check(L.moe_align_block_size(topk_ids.data_ptr(), _lib.ID_DTYPE_CODE[topk_ids.dtype], numel,
+                                     num_experts, block_size, sorted_token_ids.data_ptr(),
+                                     sorted_token_ids.numel(), experts_ids.data_ptr(),
+                                     experts_ids.numel(), num_tokens_post_pad.data_ptr(),
+                                     ws.data_ptr() if ws is not None else None,
+                                     ws.numel() if ws is not None else 0,
+                                     stream_ptr(topk_ids.device)))
+
+
+def _act_args(out: torch.Tensor, input: torch.Tensor):
+    require_gpu_tensor(input, "input")
+    if input.dtype not in _lib.DTYPE_CODE:
+        raise RuntimeError(f"activation kernel not implemented for '{input.dtype}'")
+    if out.dtype != input.dtype:
+        raise RuntimeError("out and input must have the same dtype")
+    if not (out.is_contiguous() and input.is_contiguous()):
+        raise RuntimeError("out and input must be contiguous")
+    d = input.size(-1) // 2
+    rows = input.numel() // (2 * d) if d else 0
+    if out.numel() != rows * d:
+        raise RuntimeError("out must have shape [..., d] for input [..., 2 * d]")
+    return rows, d
+
+
+def silu_and_mul(out: torch.Tensor, input: torch.Tensor) -> None:
+    """csrc/activation_kernels.cu:68-87: out = silu(input[..., :d]) * input[..., d:]."""
+    rows, d = _act_args(out, input)
+    with torch.cuda.device(input.device):
+        check(lib().moe_silu_and_mul(out.data_ptr(), input.data_ptr(), rows, d,
+                                     _lib.DTYPE_CODE[input.dtype], stream_ptr(input.device)))
+
+
+def swigluoai_and_mul(out: torch.Tensor, input: torch.Tensor, alpha: float = 1.702,
+                      limit: float = 7.0) -> None:
+    """csrc/activation_kernels.cu:89-109 (gate/up interleaved)."""
+    rows, d = _act_args(out, input)
+    with torch.cuda.device(input.device):
+        check(lib().moe_swigluoai_and_mul(out.data_ptr(), input.data_ptr(), rows, d,
+                                          _lib.DTYPE_CODE[input.dtype], alpha, limit,
+                                          stream_ptr(input.device)))
+
+
+def moe_sum(input: torch.Tensor, output: torch.Tensor) -> None:
+    """nanovllm/layers/for_moe/moe_easy_kernel.py:26-31: output = input.sum(dim=1)."""
+    require_gpu_tensor(input, "input")
+    if input.dim() != 3 or output.dim() != 2:
+        raise RuntimeError("moe_sum: input must be [T, K, H] and output [T, H]")
+    T, K, H = input.shape
+    if tuple(output.shape) != (T, H) or output.dtype != input.dtype:
+        raise RuntimeError("moe_sum: output must be [T, H] of the input dtype")
+    if not (input.is_contiguous() and output.is_contiguous()):
+        raise RuntimeError("moe_sum: tensors must be contiguous")
+    if input.dtype not in _lib.DTYPE_CODE:
+        raise RuntimeError(f"moe_sum not implemented for '{input.dtype}'")
+    with torch.cuda.device(input.device):
+        check(lib().moe_sum(output.data_ptr(), input.data_ptr(), T, K, H,
+                            _lib.DTYPE_CODE[input.dtype], stream_ptr(input.device)))
+
+
+def quant_rows_e4m3(w: torch.Tensor):
+    """[..., cols] -> (e4m3fn codes as uint8 of the same shape, fp32 scales [...]):
+    per-row s = amax|w| / 448.  No counterpart in the reference."""
+    require_gpu_tensor(w, "w")
+    if w.dtype not in _lib.DTYPE_CODE or not w.is_contiguous():
+        raise RuntimeError("quant_rows_e4m3: contiguous fp32/fp16/bf16 tensor expected")
+    cols = w.size(-1)
+    rows = w.numel() // cols
+    q = torch.empty(w.shape, dtype=torch.uint8, device=w.device)
+    s = torch.empty(w.shape[:-1], dtype=torch.float32, device=w.device)
+    with torch.cuda.device(w.device):
+        check(lib().moe_quant_rows_e4m3(w.data_ptr(), _lib.DTYPE_CODE[w.dtype], rows, cols,
+                                        q.data_ptr(), s.data_ptr(), stream_ptr(w.device)))
+    return q, s

@@ -1,0 +1,193 @@
+"""GPU parity of the expert MLP (grouped GEMMs, fused activation, combine) and
+of the stand-alone activation / combine ops against the CPU oracle."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+# tolerances of the north star: bf16 results against the fp32 oracle
+RTOL, ATOL = 2e-2, 1e-2
+
+
+def _layer(E, H, I, T, K, seed, dtype, wstd=0.05):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    w13 = (torch.randn(E, 2 * I, H, generator=g) * wstd).to(dtype)
+    w2 = (torch.randn(E, H, I, generator=g) * wstd).to(dtype)
+    logits = torch.randn(T, E, generator=g)
+    return x, w13, w2, logits
+
+
+def _close(got, want, rtol=RTOL, atol=ATOL):
+    got, want = got.float().cpu(), want.float()
+    bad = (got - want).abs() > atol + rtol * want.abs()
+    assert not bad.any(), f"{bad.sum().item()} of {bad.numel()} off; max abs err {(got - want).abs().max().item():.4g}"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("E,H,I,T,K", [(8, 256, 128, 64, 2), (4, 64, 64, 1, 1), (16, 512, 192, 300, 4),
+                                       (8, 128, 96, 777, 2), (128, 512, 256, 256, 8),
+                                       (3, 72, 40, 50, 2)])
+def test_fused_experts_against_oracle(moe, oracle, dev, dtype, E, H, I, T, K):
+    print(f"fused_experts {dtype} E={E} H={H} I={I} T={T} K={K}", flush=True)
+    x, w13, w2, logits = _layer(E, H, I, T, K, 17 + E + T, dtype)
+    tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
+    out = moe.fused_experts(x.to(dev), w13.to(dev), w2.to(dev), None, None, tw.to(dev), ids.to(dev))
+    torch.cuda.synchronize()
+    assert out.dtype == dtype and out.shape == x.shape
+    _close(out, oracle.fused_experts_ref(x, w13, w2, tw, ids))
+    # against the oracle that rounds where the reference stores intermediates the
+    # agreement is much tighter (only the fp32 summation order differs)
+    mirrored = oracle.fused_experts_ref(x, w13, w2, tw, ids, mirror_rounding=True)
+    _close(out, mirrored, rtol=1.6e-2, atol=2e-3)
+
+
+@pytest.mark.parametrize("bm", [32, 64, 128])
+def test_every_block_size_kernel(moe, oracle, dev, bm, monkeypatch):
+    x, w13, w2, logits = _layer(16, 256, 128, 500, 4, 5, torch.bfloat16)
+    tw, ids, _ = oracle.topk_softmax(logits, 4, renormalize=True)
+    monkeypatch.setattr(moe.fused_moe, "try_get_optimal_moe_config",
+                        lambda *a, **k: {"BLOCK_SIZE_M": bm})
+    out = moe.fused_experts(x.to(dev), w13.to(dev), w2.to(dev), None, None, tw.to(dev), ids.to(dev))
+    _close(out, oracle.fused_experts_ref(x, w13, w2, tw, ids))
+
+
+def test_inplace_aliases_input_and_matches(moe, oracle, dev):
+    x, w13, w2, logits = _layer(8, 256, 128, 200, 2, 9, torch.bfloat16)
+    tw, ids, _ = oracle.topk_softmax(logits, 2, renormalize=True)
+    xd = x.to(dev)
+    ref = moe.fused_experts(xd.clone(), w13.to(dev), w2.to(dev), None, None, tw.to(dev), ids.to(dev))
+    out = moe.fused_experts(xd, w13.to(dev), w2.to(dev), None, None, tw.to(dev), ids.to(dev), inplace=True)
+    assert out.data_ptr() == xd.data_ptr()
+    assert torch.equal(out, ref)
+
+
+def test_bias_router_weight_on_input_and_other_activations(moe, oracle, dev):
+    E, H, I, T, K = 8, 128, 64, 150, 1
+    x, w13, w2, logits = _layer(E, H, I, T, K, 21, torch.bfloat16)
+    g = torch.Generator().manual_seed(2)
+    b13 = (torch.randn(E, 2 * I, generator=g) * 0.1).bfloat16()
+    b2 = (torch.randn(E, H, generator=g) * 0.1).bfloat16()
+    tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=False)
+    d = lambda t: t.to(dev)
+    for act in ("silu", "swigluoai", "gelu"):
+        for on_input in (False, True):
+            out = moe.fused_experts(d(x), d(w13), d(w2), d(b13), d(b2), d(tw), d(ids), activation=act,
+                                    apply_router_weight_on_input=on_input)
+            ref = oracle.fused_experts_ref(x, w13, w2, tw, ids, activation=act, w1_bias=b13, w2_bias=b2,
+                                           apply_router_weight_on_input=on_input, mirror_rounding=True)
+            _close(out, ref, rtol=2e-2, atol=4e-3)
+    with pytest.raises(ValueError, match="Unsupported FusedMoe activation"):
+        moe.fused_experts(d(x), d(w13), d(w2), None, None, d(tw), d(ids), activation="relu")
+
+
+def test_strided_expert_weights(moe, oracle, dev):
+    # w13 / w2 as views with a padded row stride (last dimension contiguous)
+    E, H, I, T, K = 4, 128, 64, 90, 2
+    x, w13, w2, logits = _layer(E, H, I, T, K, 33, torch.bfloat16)
+    tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
+    big13 = torch.zeros(E, 2 * I, H + 64, dtype=torch.bfloat16, device=dev)
+    big13[:, :, :H] = w13.to(dev)
+    big2 = torch.zeros(E, H, I + 8, dtype=torch.bfloat16, device=dev)
+    big2[:, :, :I] = w2.to(dev)
+    out = moe.fused_experts(x.to(dev), big13[:, :, :H], big2[:, :, :I], None, None, tw.to(dev), ids.to(dev))
+    _close(out, oracle.fused_experts_ref(x, w13, w2, tw, ids))
+
+
+def test_linearity_and_permutation_properties_at_full_decode_size(moe, oracle, dev):
+    wl = moe.workloads
+    shape, x, logits, w13, w2 = wl.make_config("decode_256")
+    d = lambda t: t.to(dev)
+    tw, ids, _ = moe.fused_topk(d(x), d(logits), shape.top_k, True)
+    a = moe.fused_experts(d(x), d(w13), d(w2), None, None, tw, ids)
+    perm = torch.randperm(x.shape[0], generator=torch.Generator().manual_seed(0)).to(dev)
+    b = moe.fused_experts(d(x)[perm].contiguous(), d(w13), d(w2), None, None, tw[perm].contiguous(),
+                          ids[perm].contiguous())
+    _close(b, a[perm].cpu(), rtol=1e-2, atol=2e-3)
+    z = moe.fused_experts(d(x), d(w13), d(w2), None, None, torch.zeros_like(tw), ids)
+    assert torch.count_nonzero(z) == 0
+    # sampled rows against the fp32 oracle
+    rows = torch.arange(0, x.shape[0], 8)
+    ref = oracle.fused_experts_ref(x[rows], w13, w2, tw.cpu()[rows], ids.cpu()[rows])
+    _close(a[rows.to(dev)], ref)
+
+
+def test_layered_prefill_batch_sampled_rows(moe, oracle, dev):
+    """Config 3 (8192 prefill + 256 decode tokens): every row is independent of
+    the others, so a sample of rows is checked against the fp32 oracle."""
+    wl = moe.workloads
+    shape, x, logits, w13, w2 = wl.make_config("layered_8192p_256d")
+    d = lambda t: t.to(dev)
+    w13d, w2d = d(w13), d(w2)
+    tw, ids, _ = moe.fused_topk(d(x), d(logits), shape.top_k, True)
+    out = moe.fused_experts(d(x), w13d, w2d, None, None, tw, ids)
+    torch.cuda.synchronize()
+    rows = torch.cat([torch.arange(0, 8192, 257), torch.arange(8192, 8448, 31)])
+    ref = oracle.fused_experts_ref(x[rows], w13, w2, tw.cpu()[rows], ids.cpu()[rows])
+    _close(out[rows.to(dev)], ref)
+    # chunked prefill (16 x (512 + 256)) gives the same rows as the single pass
+    dec = slice(8192, 8448)
+    for c in (0, 7, 15):
+        sel = torch.cat([torch.arange(c * 512, (c + 1) * 512), torch.arange(8192, 8448)]).to(dev)
+        part = moe.fused_experts(d(x)[sel].contiguous(), w13d, w2d, None, None, tw[sel].contiguous(),
+                                 ids[sel].contiguous())
+        _close(part, out[sel].cpu(), rtol=1e-2, atol=2e-3)
+
+
+def test_fused_moe_module_forward(moe, oracle, dev):
+    wl = moe.workloads
+    shape, x, logits, w13, w2 = wl.make_config("tiny_fp32")
+    layer = moe.FusedMoE(shape.experts, shape.top_k, shape.hidden, shape.intermediate,
+                         params_dtype=torch.bfloat16, renormalize=True).to(dev)
+    assert tuple(layer.w13_weight.shape) == (8, 256, 256) and tuple(layer.w2_weight.shape) == (8, 256, 128)
+    layer.w13_weight.data.copy_(w13)
+    layer.w2_weight.data.copy_(w2)
+    xb = x.bfloat16()
+    hs = xb.to(dev)
+    out = layer(hs, logits.to(dev))
+    assert out.data_ptr() == hs.data_ptr()  # inplace=True, as the reference's apply()
+    tw, ids, _ = oracle.fused_topk(xb, logits, shape.top_k, True)
+    ref = oracle.fused_experts_ref(xb, w13.bfloat16(), w2.bfloat16(), tw, ids)
+    _close(out, ref)
+
+
+# ------------------------------------------------------------------ element-wise ops
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,d", [(1, 8), (5, 768), (300, 96), (17, 7)])
+def test_silu_and_mul_bit_exact(moe, oracle, dev, dtype, rows, d):
+    x = (torch.randn(rows, 2 * d, generator=torch.Generator().manual_seed(rows + d)) * 4).to(dtype)
+    out = torch.empty(rows, d, dtype=dtype, device=dev)
+    moe.ops.silu_and_mul(out, x.to(dev))
+    want = oracle.silu_and_mul(x)
+    assert torch.equal(out.cpu().view(torch.int16 if dtype != torch.float32 else torch.int32),
+                       want.view(torch.int16 if dtype != torch.float32 else torch.int32))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swigluoai_and_mul_bit_exact(moe, oracle, dev, dtype):
+    x = (torch.randn(40, 2 * 360, generator=torch.Generator().manual_seed(1)) * 5).to(dtype)
+    out = torch.empty(40, 360, dtype=dtype, device=dev)
+    moe.ops.swigluoai_and_mul(out, x.to(dev), 1.702, 7.0)
+    want = oracle.swigluoai_and_mul(x, 1.702, 7.0)
+    assert torch.equal(out.cpu().view(torch.int16 if dtype != torch.float32 else torch.int32),
+                       want.view(torch.int16 if dtype != torch.float32 else torch.int32))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_moe_sum(moe, dev, dtype):
+    x = torch.randn(33, 8, 200, generator=torch.Generator().manual_seed(3)).to(dtype)
+    out = torch.empty(33, 200, dtype=dtype, device=dev)
+    moe.ops.moe_sum(x.to(dev), out)
+    want = x.float().sum(1)
+    assert torch.allclose(out.cpu().float(), want, rtol=2 ** -7 if dtype != torch.float32 else 1e-6, atol=1e-5)
+
+
+def test_quant_rows_e4m3_matches_oracle(moe, oracle, dev):
+    w = torch.randn(64, 512, generator=torch.Generator().manual_seed(7)) * 0.02
+    w[3] = 0
+    for dtype in (torch.float32, torch.bfloat16):
+        wd = w.to(dtype)
+        q, s = moe.ops.quant_rows_e4m3(wd.to(dev))
+        oq, os_ = oracle.quant_weight_per_channel(wd[None])
+        assert torch.equal(s.cpu(), os_[0])
+        assert torch.equal(q.cpu(), oq[0])

@@ -1,0 +1,157 @@
+"""GPU parity, bit-exact: router softmax/top-k and expert-sorted alignment
+through the C ABI (via the Python ops) against the CPU oracle."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_topk(moe, g, K, renorm, dev):
+    T = g.shape[0]
+    w = torch.full((T, K), -7.0, dtype=torch.float32, device=dev)
+    ids = torch.full((T, K), -7, dtype=torch.int32, device=dev)
+    tei = torch.full((T, K), -7, dtype=torch.int32, device=dev)
+    moe.ops.topk_softmax(w, ids, tei, g.to(dev), renormalize=renorm)
+    torch.cuda.synchronize()
+    return w.cpu(), ids.cpu(), tei.cpu()
+
+
+@pytest.mark.parametrize("E", [1, 2, 4, 8, 16, 32, 64, 128, 256, 3, 48, 100, 384, 1000, 1024])
+@pytest.mark.parametrize("T", [1, 7, 257])
+def test_topk_softmax_bit_exact(moe, oracle, dev, E, T):
+    print(f"topk_softmax E={E} T={T}", flush=True)
+    g = torch.randn(T, E, generator=torch.Generator().manual_seed(E * 1000 + T)) * 2
+    for K in sorted({1, min(2, E), min(8, E), E if E <= 16 else min(8, E)}):
+        for renorm in (False, True):
+            w, ids, tei = _run_topk(moe, g, K, renorm, dev)
+            ow, oids, otei = oracle.topk_softmax(g, K, renormalize=renorm)
+            assert torch.equal(ids, oids), (E, T, K, renorm)
+            assert torch.equal(tei, otei)
+            assert torch.equal(w.view(torch.int32), ow.view(torch.int32)), (E, T, K, renorm)
+
+
+def test_topk_softmax_ties_and_bf16_logits(moe, oracle, dev):
+    g = torch.zeros(130, 128)
+    w, ids, _ = _run_topk(moe, g, 8, False, dev)
+    assert torch.equal(ids, torch.arange(8, dtype=torch.int32).repeat(130, 1))
+    gq = torch.randn(4096, 128, generator=torch.Generator().manual_seed(3)).bfloat16().float()
+    for renorm in (False, True):
+        w, ids, tei = _run_topk(moe, gq, 8, renorm, dev)
+        ow, oids, otei = oracle.topk_softmax(gq, 8, renormalize=renorm)
+        assert torch.equal(ids, oids) and torch.equal(w.view(torch.int32), ow.view(torch.int32))
+
+
+def test_topk_softmax_extreme_logits(moe, oracle, dev):
+    g = torch.randn(64, 128, generator=torch.Generator().manual_seed(8)) * 40
+    g[0, :] = -1e4
+    g[1, 5] = 1e4
+    w, ids, tei = _run_topk(moe, g, 8, True, dev)
+    ow, oids, otei = oracle.topk_softmax(g, 8, renormalize=True)
+    assert torch.equal(ids, oids) and torch.equal(w.view(torch.int32), ow.view(torch.int32))
+
+
+def test_fused_topk_matches_oracle_at_full_size(moe, oracle, dev):
+    shape, x, logits, _, _ = None, None, None, None, None
+    wl = moe.workloads
+    x, logits = wl.make_inputs(wl.QWEN3_30B_A3B, 8448, 2, torch.bfloat16)
+    w, ids, tei = moe.fused_topk(x.to(dev), logits.to(dev), 8, True)
+    ow, oids, otei = oracle.fused_topk(x, logits, 8, True)
+    assert torch.equal(ids.cpu(), oids) and torch.equal(tei.cpu(), otei)
+    assert torch.equal(w.cpu().view(torch.int32), ow.view(torch.int32))
+    # bf16 router logits (what the model hands over) are upcast, ties and all
+    w2, ids2, _ = moe.fused_topk(x.to(dev), logits.bfloat16().to(dev), 8, True)
+    ow2, oids2, _ = oracle.fused_topk(x, logits.bfloat16().float(), 8, True)
+    assert torch.equal(ids2.cpu(), oids2) and torch.equal(w2.cpu().view(torch.int32), ow2.view(torch.int32))
+
+
+def test_topk_softmax_rejects_bad_arguments(moe, dev):
+    g = torch.zeros(4, 8, device=dev)
+    w = torch.empty(4, 9, device=dev)
+    i = torch.empty(4, 9, dtype=torch.int32, device=dev)
+    with pytest.raises(RuntimeError, match="exceeds num_experts"):
+        moe.ops.topk_softmax(w, i, i.clone(), g)
+    with pytest.raises(RuntimeError, match="Float"):
+        moe.ops.topk_softmax(w[:, :2].contiguous(), i[:, :2].contiguous(), i[:, :2].contiguous(), g.half())
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        moe.ops.topk_softmax(w.cpu(), i.cpu(), i.cpu(), g.cpu())
+
+
+# ------------------------------------------------------------------ alignment
+ALIGN_CASES = [
+    (0, 8, 16), (1, 1, 1), (9, 5, 4), (12, 5, 4), (128, 8, 64), (2048, 128, 16), (2048, 128, 32),
+    (2048, 128, 64), (2048, 128, 128), (6144, 128, 64), (16384, 128, 32), (16385, 128, 32),
+    (67584, 128, 64), (67584, 128, 128), (67584, 128, 16), (524288, 128, 128), (30000, 60, 7),
+    (5000, 1000, 16), (70000, 1024, 8), (3000, 600, 32), (40000, 512, 64), (1000, 2, 256),
+]
+
+
+def _skewed_ids(numel, E, seed):
+    g = torch.Generator().manual_seed(seed)
+    if numel == 0:
+        return torch.zeros(0, dtype=torch.int32)
+    p = torch.arange(1, E + 1, dtype=torch.float64) ** -1.1
+    p = p[torch.randperm(E, generator=g)]
+    return torch.multinomial(p, numel, replacement=True, generator=g).to(torch.int32)
+
+
+@pytest.mark.parametrize("numel,E,bm", ALIGN_CASES)
+def test_moe_align_block_size_bit_exact(moe, oracle, dev, numel, E, bm):
+    print(f"align numel={numel} E={E} bm={bm}", flush=True)
+    ids = _skewed_ids(numel, E, numel + 7 * E + bm)
+    s, e, n = moe.moe_align_block_size(ids.to(dev), bm, E)
+    torch.cuda.synchronize()
+    os_, oe, on = oracle.moe_align_block_size(ids, bm, E)
+    assert n.cpu().item() == on.item()
+    assert torch.equal(e.cpu(), oe)
+    assert torch.equal(s.cpu(), os_)
+
+
+@pytest.mark.parametrize("dtype", [torch.int32, torch.int64, torch.int16, torch.uint8, torch.int8])
+def test_moe_align_block_size_id_dtypes_and_out_of_range_ids(moe, oracle, dev, dtype):
+    E = 100
+    ids = torch.randint(0, 120, (20000,), generator=torch.Generator().manual_seed(4))  # ids >= E dropped
+    if dtype != torch.uint8:
+        ids[::97] = -3
+    else:
+        ids = ids.clamp(min=0)
+    ids = ids.to(dtype)
+    for n_take in (20000, 3000):
+        s, e, n = moe.moe_align_block_size(ids[:n_take].to(dev), 32, E)
+        os_, oe, on = oracle.moe_align_block_size(ids[:n_take], 32, E)
+        assert torch.equal(s.cpu(), os_) and torch.equal(e.cpu(), oe) and n.cpu().item() == on.item()
+
+
+def test_moe_align_known_answers_from_reference_comments(moe, dev):
+    ids = torch.tensor([[2, 3, 4], [1, 2, 4], [1, 3, 4], [1, 2, 3]], dtype=torch.int32, device=dev)
+    s, e, n = moe.moe_align_block_size(ids, 4, 5)
+    assert s[:16].tolist() == [3, 6, 9, 12, 0, 4, 10, 12, 1, 7, 11, 12, 2, 5, 8, 12]
+    assert n.item() == 16 and e[:4].tolist() == [1, 2, 3, 4]
+    ids = torch.tensor([0, 1, 2, 1, 2, 3, 0, 3, 4], dtype=torch.int32, device=dev)
+    s, e, n = moe.moe_align_block_size(ids, 4, 5)
+    assert s[:20].tolist() == [0, 6, 9, 9, 1, 3, 9, 9, 2, 4, 9, 9, 5, 7, 9, 9, 8, 9, 9, 9]
+    assert n.item() == 20
+
+
+def test_alignment_is_deterministic_and_routed_config_matches(moe, oracle, dev):
+    wl = moe.workloads
+    x, logits = wl.make_inputs(wl.QWEN3_30B_A3B, 8448, 2, torch.bfloat16)
+    _, ids, _ = moe.fused_topk(x.to(dev), logits.to(dev), 8, True)
+    first = moe.moe_align_block_size(ids, 128, 128)
+    for _ in range(3):
+        again = moe.moe_align_block_size(ids, 128, 128)
+        assert all(torch.equal(a, b) for a, b in zip(first, again))
+    want = oracle.moe_align_block_size(ids.cpu(), 128, 128)
+    assert all(torch.equal(a.cpu(), b) for a, b in zip(first, want))
+
+
+def test_ops_level_align_signature(moe, oracle, dev):
+    ids = _skewed_ids(700, 16, 1).to(dev)
+    P = 700 + 16 * 31
+    s = torch.empty(P, dtype=torch.int32, device=dev)
+    e = torch.empty((P + 31) // 32, dtype=torch.int32, device=dev)
+    n = torch.empty(1, dtype=torch.int32, device=dev)
+    moe.ops.moe_align_block_size(ids, 16, 32, s, e, n)
+    os_, oe, on = oracle.moe_align_block_size(ids.cpu(), 32, 16)
+    assert torch.equal(s.cpu(), os_) and torch.equal(e.cpu(), oe) and n.item() == on.item()
+    with pytest.raises(RuntimeError, match="holds"):
+        moe.ops.moe_align_block_size(ids, 16, 32, s[:100].contiguous(), e, n)

@@ -1,0 +1,332 @@
+"""Pins the CPU oracle: known answers from the reference's comments, closed
+forms, library routines on special cases and brute force on tiny inputs."""
+import math
+
+import numpy as np
+import pytest
+import torch
+from hypothesis import given, settings, strategies as st
+
+
+# ----------------------------------------------------------------- exp
+def test_expf_within_2ulp_of_float64(oracle):
+    x = torch.cat([torch.linspace(-87, 0, 200001), torch.linspace(0, 88, 100001),
+                   torch.tensor([0.0, -0.0, 1e-8, -1e-8, -86.999, 87.999])]).float()
+    y = oracle.expf(x).double().numpy()
+    ref = np.exp(x.double().numpy())
+    ulp = np.spacing(ref.astype(np.float32)).astype(np.float64)
+    err = np.abs(y - ref) / ulp
+    assert err.max() <= 2.0, err.max()
+
+
+def test_expf_special_values(oracle):
+    x = torch.tensor([0.0, -100.0, -87.5, 89.0, float("inf"), float("-inf"), float("nan")])
+    y = oracle.expf(x)
+    assert y[0] == 1.0 and y[1] == 0.0 and y[2] == 0.0
+    assert math.isinf(y[3]) and math.isinf(y[4]) and y[5] == 0.0 and math.isnan(y[6])
+
+
+def test_expf_is_monotone_on_softmax_range(oracle):
+    x = torch.linspace(-30, 0, 2_000_001).float()
+    y = oracle.expf(x)
+    assert bool((y[1:] >= y[:-1]).all())
+
+
+# ----------------------------------------------------------------- router
+def _softmax64(g):
+    return torch.softmax(g.double(), -1)
+
+
+@pytest.mark.parametrize("E,K", [(1, 1), (2, 1), (4, 2), (8, 2), (16, 4), (32, 8), (64, 6),
+                                 (128, 8), (256, 8), (3, 2), (48, 4), (100, 8), (384, 8),
+                                 (1000, 5)])
+def test_topk_softmax_against_float64_softmax(oracle, E, K):
+    g = torch.randn(37, E, generator=torch.Generator().manual_seed(E * 31 + K))
+    w, ids, tei, probs = oracle.topk_softmax(g, K, return_probs=True)
+    p64 = _softmax64(g)
+    assert torch.allclose(probs.double(), p64, rtol=2e-6, atol=1e-12)
+    # each weight is the probability of its expert; ids distinct; weights non-increasing
+    assert torch.equal(w, torch.gather(probs, 1, ids.long()))
+    assert all(len(set(r.tolist())) == K for r in ids)
+    assert bool((w[:, 1:] <= w[:, :-1]).all())
+    # ids are the stable descending order of the probabilities
+    order = torch.argsort(probs, dim=-1, descending=True, stable=True)[:, :K]
+    assert torch.equal(ids.long(), order)
+    T = g.shape[0]
+    expect_tei = torch.arange(K)[None, :] * T + torch.arange(T)[:, None]
+    assert torch.equal(tei.long(), expect_tei)
+
+
+def test_topk_softmax_ids_follow_logits_when_probabilities_distinct(oracle):
+    g = torch.randn(512, 128, generator=torch.Generator().manual_seed(5))
+    w, ids, _, probs = oracle.topk_softmax(g, 8, return_probs=True)
+    sp = torch.sort(probs, dim=-1, descending=True).values
+    distinct = (sp[:, :9][:, 1:] != sp[:, :9][:, :-1]).all(dim=1)
+    assert distinct.float().mean() > 0.9
+    by_logit = torch.argsort(g, dim=-1, descending=True, stable=True)[:, :8]
+    assert torch.equal(ids.long()[distinct], by_logit[distinct])
+
+
+def test_topk_softmax_ties_take_lowest_index(oracle):
+    g = torch.zeros(3, 16)
+    w, ids, _ = oracle.topk_softmax(g, 4)
+    assert torch.equal(ids, torch.arange(4, dtype=torch.int32).repeat(3, 1))
+    assert torch.equal(w, torch.full((3, 4), 1.0 / 16))
+    # bf16-quantised logits produce many exact ties
+    gq = torch.randn(200, 128, generator=torch.Generator().manual_seed(9)).bfloat16().float()
+    gq = (gq * 4).round() / 4
+    w, ids, _, probs = oracle.topk_softmax(gq, 8, return_probs=True)
+    order = torch.argsort(probs, dim=-1, descending=True, stable=True)[:, :8]
+    assert torch.equal(ids.long(), order)
+    # a tie that straddles the cut: the lower expert index must be kept
+    for r in range(gq.shape[0]):
+        kth = probs[r, ids[r, -1].long()]
+        tied = torch.nonzero(probs[r] == kth).flatten()
+        chosen = [i for i in ids[r].tolist() if probs[r, i] == kth]
+        assert chosen == tied[:len(chosen)].tolist()
+
+
+def test_topk_softmax_k1_is_argmax_and_kE_is_full_sort(oracle):
+    g = torch.randn(50, 32, generator=torch.Generator().manual_seed(3))
+    _, ids, _ = oracle.topk_softmax(g, 1)
+    assert torch.equal(ids.flatten().long(), g.argmax(-1))
+    w, ids, _ = oracle.topk_softmax(g, 32)
+    assert torch.equal(ids.long(), torch.argsort(g, dim=-1, descending=True, stable=True))
+    assert torch.allclose(w.sum(-1), torch.ones(50), atol=1e-6)
+
+
+def test_topk_softmax_brute_force_tiny(oracle):
+    rng = np.random.default_rng(0)
+    for E in (2, 3, 4, 5, 8):
+        for _ in range(40):
+            g = rng.integers(-3, 4, size=(1, E)).astype(np.float32) / 2
+            K = int(rng.integers(1, E + 1))
+            w, ids, _ = oracle.topk_softmax(torch.from_numpy(g), K)
+            ex = [math.exp(float(v) - float(g.max())) for v in g[0]]
+            p = [v / sum(ex) for v in ex]
+            pool = list(range(E))
+            want = []
+            for _k in range(K):
+                best = max(pool, key=lambda i: (round(p[i], 9), -i))
+                want.append(best)
+                pool.remove(best)
+            assert ids[0].tolist() == want
+            assert np.allclose(w[0].numpy(), [p[i] for i in want], rtol=1e-6)
+
+
+def test_renormalised_weights_equal_softmax_over_selected_logits(oracle):
+    # identity used by the reference's unused torch stand-in
+    # (nanovllm/layers/for_moe/moe_easy_kernel.py:17-19)
+    g = torch.randn(64, 128, generator=torch.Generator().manual_seed(11))
+    w, ids, _ = oracle.topk_softmax(g, 8, renormalize=True)
+    sel = torch.gather(g, 1, ids.long())
+    assert torch.allclose(w.double(), torch.softmax(sel.double(), -1), rtol=1e-5)
+    assert torch.allclose(w.sum(-1), torch.ones(64), atol=1e-6)
+    w_raw, _, _ = oracle.topk_softmax(g, 8, renormalize=False)
+    s = torch.zeros(64)
+    for k in range(8):
+        s = s + w_raw[:, k]
+    assert torch.equal(w, w_raw / s[:, None])
+
+
+def test_topk_rejects_k_above_e(oracle):
+    with pytest.raises(ValueError):
+        oracle.topk_softmax(torch.zeros(2, 4), 5)
+
+
+# ----------------------------------------------------------------- alignment
+def test_align_known_answer_python_docstring(oracle):
+    # nanovllm/layers/for_moe/fused_moe.py:42-55 (ids reach 4, so five experts)
+    ids = torch.tensor([[2, 3, 4], [1, 2, 4], [1, 3, 4], [1, 2, 3]], dtype=torch.int32)
+    s, e, n = oracle.moe_align_block_size(ids, 4, 5)
+    assert s[:16].tolist() == [3, 6, 9, 12, 0, 4, 10, 12, 1, 7, 11, 12, 2, 5, 8, 12]
+    assert n.item() == 16 and e[:4].tolist() == [1, 2, 3, 4]
+    assert set(s[16:].tolist()) == {12} and set(e[4:].tolist()) <= {0}
+
+
+def test_align_known_answer_cuda_comment(oracle):
+    # csrc/moe_align_block_size_kernels.cu:92-95
+    ids = torch.tensor([0, 1, 2, 1, 2, 3, 0, 3, 4], dtype=torch.int32)
+    s, e, n = oracle.moe_align_block_size(ids, 4, 5)
+    P = 9
+    assert s[:20].tolist() == [0, 6, P, P, 1, 3, P, P, 2, 4, P, P, 5, 7, P, P, 8, P, P, P]
+    assert n.item() == 20 and e[:5].tolist() == [0, 1, 2, 3, 4]
+
+
+def _align_numpy(ids, bm, E):
+    ids = np.asarray(ids).reshape(-1)
+    numel = ids.size
+    valid = (ids >= 0) & (ids < E)
+    order = np.argsort(np.where(valid, ids, E), kind="stable")
+    order = order[: valid.sum()]
+    cnt = np.bincount(ids[valid], minlength=E)
+    pad = (cnt + bm - 1) // bm * bm
+    cum = np.concatenate([[0], np.cumsum(pad)])
+    P = numel + E * (bm - 1)
+    out = np.full(P, numel, dtype=np.int32)
+    off = 0
+    for e in range(E):
+        out[cum[e]:cum[e] + cnt[e]] = order[off:off + cnt[e]]
+        off += cnt[e]
+    B = (P + bm - 1) // bm
+    eid = np.zeros(B, dtype=np.int32)
+    for e in range(E):
+        eid[cum[e] // bm: cum[e + 1] // bm] = e
+    return out, eid, int(cum[-1])
+
+
+@pytest.mark.parametrize("numel,E,bm", [(0, 4, 4), (1, 1, 1), (9, 5, 4), (128, 8, 64),
+                                        (2048, 128, 16), (2048, 128, 64), (5000, 60, 32),
+                                        (67584, 128, 128), (3000, 1000, 16)])
+def test_align_equals_numpy_stable_argsort(oracle, numel, E, bm):
+    rng = np.random.default_rng(numel + E)
+    ids = rng.integers(0, E, size=numel).astype(np.int32)
+    s, e, n = oracle.moe_align_block_size(torch.from_numpy(ids), bm, E)
+    ws, we, wn = _align_numpy(ids, bm, E)
+    assert n.item() == wn
+    assert np.array_equal(s.numpy(), ws) and np.array_equal(e.numpy(), we)
+
+
+@settings(max_examples=150, deadline=None)
+@given(st.integers(1, 6), st.integers(1, 5), st.lists(st.integers(-1, 7), max_size=40))
+def test_align_invariants_brute_force(E, bm, raw):
+    import importlib
+    oracle = importlib.import_module("oracle.moe_oracle")
+    ids = torch.tensor(raw, dtype=torch.int64)
+    numel = len(raw)
+    s, e, n = oracle.moe_align_block_size(ids, bm, E)
+    s, e, n = s.tolist(), e.tolist(), n.item()
+    cnt = [sum(1 for v in raw if v == x) for x in range(E)]
+    assert n == sum((c + bm - 1) // bm * bm for c in cnt)
+    assert all(v == numel for v in s[n:]) and all(v == 0 for v in e[n // bm:])
+    real = [v for v in s[:n] if v != numel]
+    assert sorted(real) == [i for i, v in enumerate(raw) if 0 <= v < E]
+    for b in range(n // bm):
+        blk = s[b * bm:(b + 1) * bm]
+        toks = [v for v in blk if v != numel]
+        assert all(raw[t] == e[b] for t in toks)
+        assert toks == sorted(toks)
+        assert blk[:len(toks)] == toks  # real ids first, then padding
+    pos = {v: i for i, v in enumerate(s[:n]) if v != numel}
+    for x in range(E):
+        mine = [i for i, v in enumerate(raw) if v == x]
+        assert [pos[i] for i in mine] == sorted(pos[i] for i in mine)
+
+
+@pytest.mark.parametrize("dtype", [torch.int32, torch.int64, torch.int16, torch.int8, torch.uint8])
+def test_align_id_dtypes_agree(oracle, dtype):
+    ids = torch.randint(0, 100, (777,), generator=torch.Generator().manual_seed(1))
+    a = oracle.moe_align_block_size(ids.to(torch.int32), 16, 100)
+    b = oracle.moe_align_block_size(ids.to(dtype), 16, 100)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+
+
+# ----------------------------------------------------------------- activations
+def test_silu_and_mul_matches_formula(oracle):
+    x = torch.randn(33, 2 * 96, generator=torch.Generator().manual_seed(2)) * 3
+    out = oracle.silu_and_mul(x)
+    ref = torch.nn.functional.silu(x[:, :96].double()) * x[:, 96:].double()
+    assert torch.allclose(out.double(), ref, rtol=3e-6, atol=1e-7)
+    xb = x.bfloat16()
+    outb = oracle.silu_and_mul(xb)
+    refb = (torch.nn.functional.silu(xb[:, :96].float()).bfloat16() * xb[:, 96:])
+    diff = (outb.float() - refb.float()).abs()
+    assert (diff > 0).float().mean() < 0.01  # only exp's last ulp may flip a bf16 rounding
+    assert torch.allclose(outb.float(), refb.float(), rtol=2 ** -7, atol=1e-30)
+    xh = x.half()
+    outh = oracle.silu_and_mul(xh)
+    refh = (torch.nn.functional.silu(xh[:, :96].float()).half() * xh[:, 96:])
+    assert torch.allclose(outh.float(), refh.float(), rtol=2 ** -10, atol=1e-7)
+
+
+def test_swigluoai_matches_formula(oracle):
+    x = torch.randn(17, 2 * 64, generator=torch.Generator().manual_seed(4)) * 5
+    out = oracle.swigluoai_and_mul(x, 1.702, 7.0)
+    g = x[:, 0::2].double().clamp(max=7.0)
+    u = x[:, 1::2].double().clamp(-7.0, 7.0)
+    ref = (u + 1) * g * torch.sigmoid(1.702 * g)
+    assert torch.allclose(out.double(), ref, rtol=3e-6, atol=1e-6)
+
+
+# ----------------------------------------------------------------- fp8 helpers
+def test_e4m3_quantiser_matches_torch_cast_and_saturates(oracle):
+    x = torch.cat([torch.linspace(-448, 448, 100001), torch.tensor([0.0, 1e-4, 2 ** -9, 2 ** -10,
+                   0.0009765625 * 1.5, 447.9, 500.0, -1e9])]).float()
+    q = oracle.quant_e4m3(x)
+    d = oracle.dequant_e4m3(q)
+    inr = x.abs() <= 448
+    want = x[inr].to(torch.float8_e4m3fn).float()
+    assert torch.equal(d[inr], want)
+    assert d[-2] == 448.0 and d[-1] == -448.0
+    # round trip of every finite code
+    codes = torch.tensor([c for c in range(256) if (c & 0x7f) != 0x7f], dtype=torch.uint8)
+    vals = oracle.dequant_e4m3(codes)
+    again = oracle.dequant_e4m3(oracle.quant_e4m3(vals))
+    assert torch.equal(vals, again)
+
+
+def test_per_channel_and_per_token_scales(oracle):
+    w = torch.randn(3, 5, 64, generator=torch.Generator().manual_seed(6)) * 0.02
+    q, s = oracle.quant_weight_per_channel(w)
+    assert torch.allclose(s, w.abs().amax(-1) / 448)
+    deq = oracle.dequant_e4m3(q) * s[..., None]
+    assert ((deq - w).abs() <= w.abs().amax(-1, keepdim=True) * 2 ** -4 + 1e-9).all()
+
+
+# ----------------------------------------------------------------- expert MLP
+def _rand_layer(E=4, H=64, I=32, T=24, K=2, seed=0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    w13 = (torch.randn(E, 2 * I, H, generator=g) * 0.1).to(dtype)
+    w2 = (torch.randn(E, H, I, generator=g) * 0.1).to(dtype)
+    logits = torch.randn(T, E, generator=g)
+    return x, w13, w2, logits
+
+
+def test_fused_experts_k1_unit_weight_is_a_gated_mlp(oracle):
+    x, w13, w2, logits = _rand_layer(K=1)
+    ids = logits.argmax(-1, keepdim=True).int()
+    w = torch.ones(x.shape[0], 1)
+    out = oracle.fused_experts_ref(x, w13, w2, w, ids)
+    I = w2.shape[2]
+    for t in range(x.shape[0]):
+        e = ids[t, 0].item()
+        h = torch.nn.functional.linear(x[t], w13[e])
+        ref = torch.nn.functional.linear(torch.nn.functional.silu(h[:I]) * h[I:], w2[e])
+        assert torch.allclose(out[t], ref, rtol=1e-4, atol=1e-5)
+
+
+def test_fused_experts_single_expert_is_a_dense_mlp(oracle):
+    x, w13, w2, _ = _rand_layer(E=1, K=1)
+    ids = torch.zeros(x.shape[0], 1, dtype=torch.int32)
+    w = torch.full((x.shape[0], 1), 0.5)
+    out = oracle.fused_experts_ref(x, w13, w2, w, ids)
+    h = x @ w13[0].t()
+    I = w2.shape[2]
+    ref = 0.5 * ((torch.nn.functional.silu(h[:, :I]) * h[:, I:]) @ w2[0].t())
+    assert torch.allclose(out, ref, rtol=1e-4, atol=1e-5)
+
+
+def test_fused_experts_linear_in_weights_and_permutation_invariant(oracle):
+    x, w13, w2, logits = _rand_layer(T=40, K=2)
+    w, ids, _ = oracle.topk_softmax(logits, 2, renormalize=True)
+    a = oracle.fused_experts_ref(x, w13, w2, w, ids)
+    b = oracle.fused_experts_ref(x, w13, w2, 3 * w, ids)
+    assert torch.allclose(b, 3 * a, rtol=1e-5, atol=1e-6)
+    z = oracle.fused_experts_ref(x, w13, w2, torch.zeros_like(w), ids)
+    assert torch.count_nonzero(z) == 0
+    perm = torch.randperm(40, generator=torch.Generator().manual_seed(1))
+    c = oracle.fused_experts_ref(x[perm], w13, w2, w[perm], ids[perm])
+    assert torch.allclose(c, a[perm], rtol=1e-5, atol=1e-6)
+    # weight on the input side commutes for K-slot-wise linear second GEMM only when the
+    # activation is evaluated on the scaled input: just check it runs and differs
+    d = oracle.fused_experts_ref(x, w13, w2, w, ids, apply_router_weight_on_input=True)
+    assert d.shape == a.shape and not torch.allclose(d, a)
+
+
+def test_mirrored_rounding_stays_close_to_fp32(oracle):
+    x, w13, w2, logits = _rand_layer(T=32, K=2, dtype=torch.bfloat16)
+    w, ids, _ = oracle.topk_softmax(logits, 2, renormalize=True)
+    a = oracle.fused_experts_ref(x, w13, w2, w, ids)
+    b = oracle.fused_experts_ref(x, w13, w2, w, ids, mirror_rounding=True)
+    assert torch.allclose(a, b, rtol=2e-2, atol=1e-2)
