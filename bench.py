@@ -1,0 +1,236 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused-MoE expert path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one call of the whole layer path (router softmax/top-k, alignment,
+gate-up GEMM + SiLU*up, down GEMM * routed weight, top-k combine) on the
+Qwen3-30B-A3B-shaped layer (H 2048, 128 experts, I 768, top-8) with synthetic
+seeded inputs already resident in HBM.  The headline workload is the
+layered-prefill iteration: 8192 prefill + 256 decode tokens in one call.  The
+decode-only 256-token call (memory-bound) is measured in the same run and
+reported under "decode".  One JSON line goes to stdout.
+"""
+from __future__ import annotations
+
+import argparse
+import importlib
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "MoE layer TFLOP/s @8192+256 tok & decode HBM GB/s, Qwen3-30B-A3B layer"
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs (summaries under profiles/); None until measured.
+MEASURED_TRAFFIC_BYTES = {"layered_8192p_256d": None, "decode_256": None}
+
+
+def _events(n):
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+class Layer:
+    """Inputs of one workload on the GPU plus the pre-allocated scratch a
+    serving loop would reuse."""
+
+    def __init__(self, moe, name: str, dev):
+        wl = moe.workloads
+        self.moe = moe
+        self.name = name
+        self.shape, x, logits, w13, w2 = wl.make_config(name)
+        self.T = x.shape[0]
+        self.x, self.logits = x.to(dev), logits.to(dev)
+        self.w13, self.w2 = w13.to(dev), w2.to(dev)
+        self.dev = dev
+        s = self.shape
+        self.bm = moe.try_get_optimal_moe_config(self.w13.shape, self.w2.shape, s.top_k, None,
+                                                 self.T)["BLOCK_SIZE_M"]
+        ws = moe.fused_moe.fused_experts_workspace_bytes(self.T, s.hidden, s.intermediate,
+                                                         s.experts, s.top_k, self.bm, x.dtype)
+        self.workspace = torch.empty(ws, dtype=torch.uint8, device=dev)
+        self.out = torch.empty_like(self.x)
+
+    def step(self):
+        moe, s = self.moe, self.shape
+        tw, ids, _ = moe.fused_topk(self.x, self.logits, s.top_k, True)
+        return moe.fused_experts(self.x, self.w13, self.w2, None, None, tw, ids)
+
+    def step_instrumented(self, ev):
+        """Same work with an event after every stage (5 stages -> 6 events)."""
+        moe, s = self.moe, self.shape
+        fm = moe.fused_moe
+        ev[0].record()
+        tw, ids, _ = moe.fused_topk(self.x, self.logits, s.top_k, True)
+        ev[1].record()
+        sorted_ids, expert_ids, npp = fm.moe_align_block_size(ids, self.bm, s.experts)
+        ev[2].record()
+        for i, mask in enumerate((1, 2, 4)):
+            fm.launch_fused_experts(self.x, self.out, self.w13, self.w2, None, None, None, None, tw,
+                                    sorted_ids, expert_ids, npp, self.bm, workspace=self.workspace,
+                                    passes=mask)
+            ev[3 + i].record()
+        return ids
+
+    def n_active(self, ids) -> int:
+        return int(torch.unique(ids).numel())
+
+
+def time_steps(layer: Layer, steps: int, warmup: int):
+    for _ in range(warmup):
+        layer.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        layer.step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def time_stages(layer: Layer, steps: int):
+    names = ["topk_softmax", "moe_align_block_size", "gate_up_gemm_act", "down_gemm_weighted",
+             "topk_combine"]
+    per = {n: [] for n in names}
+    ids = None
+    for _ in range(steps):
+        ev = _events(6)
+        ids = layer.step_instrumented(ev)
+        torch.cuda.synchronize()
+        for i, n in enumerate(names):
+            per[n].append(ev[i].elapsed_time(ev[i + 1]))
+    return {n: statistics.fmean(v) for n, v in per.items()}, ids
+
+
+def cpu_baseline(moe, name: str, runs: int):
+    """The oracle (PyTorch fp32 restatement of the reference's MoE math; bf16
+    weights upcast per expert) on this host's cores: bounded sample."""
+    oracle = importlib.import_module("oracle.moe_oracle")
+    wl = moe.workloads
+    shape, x, logits, w13, w2 = wl.make_config(name)
+    cores = os.cpu_count() or 1
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit():
+        cores = min(cores, int(env))
+    torch.set_num_threads(cores)
+
+    def once():
+        tw, ids, _ = oracle.fused_topk(x, logits, shape.top_k, True)
+        oracle.moe_align_block_size(ids, 64, shape.experts)
+        return oracle.fused_experts_ref(x, w13, w2, tw, ids)
+
+    once()  # warm-up
+    t0 = time.perf_counter()
+    for _ in range(runs):
+        once()
+    dt = (time.perf_counter() - t0) / runs
+    return dt, torch.get_num_threads()
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="layered_8192p_256d",
+                    choices=["layered_8192p_256d", "decode_256"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-runs", type=int, default=2)
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build is the single-GPU (TP=1) expert path; it has no collectives "
+              "and measures one GPU only. Run with --gpus 1.", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback.", file=sys.stderr)
+        return 3
+    moe = importlib.import_module("layered-prefill_amd")
+    moe._lib.lib()
+    dev = torch.device("cuda:0")
+    wl = moe.workloads
+
+    main_layer = Layer(moe, a.workload, dev)
+    ms = time_steps(main_layer, a.steps, a.warmup)
+    stages, ids = time_stages(main_layer, max(5, a.steps // 2))
+    shape = main_layer.shape
+    flops = wl.layer_flops(main_layer.T, shape)
+    n_active = main_layer.n_active(ids)
+    abytes = wl.layer_bytes(main_layer.T, shape, n_active)
+    tflops = flops / (ms * 1e-3) / 1e12
+    gbs = abytes / (ms * 1e-3) / 1e9
+
+    compute_bound = a.workload == "layered_8192p_256d"
+    if compute_bound:
+        # dominant kernel: gate-up grouped GEMM, 4*T*K*H*I algorithmic flops
+        k_flops = 4 * main_layer.T * shape.top_k * shape.hidden * shape.intermediate
+        ach = k_flops / (stages["gate_up_gemm_act"] * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "kernel": "grouped_gemm_kernel<gate-up, SiLU*up epilogue>",
+                    "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(ach / PEAK_BF16_TFLOPS, 4),
+                    "kernel_ms": round(stages["gate_up_gemm_act"], 4),
+                    "traffic": MEASURED_TRAFFIC_BYTES[a.workload]}
+        value, unit, metric = tflops, "TFLOP/s", METRIC
+    else:
+        # dominant kernel: gate-up grouped GEMM streaming 2*H*I weights per active expert
+        k_bytes = n_active * 2 * shape.hidden * shape.intermediate * 2 + main_layer.T * shape.hidden * 2
+        ach = k_bytes / (stages["gate_up_gemm_act"] * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": "grouped_gemm_kernel<gate-up, SiLU*up epilogue>",
+                    "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(ach / PEAK_HBM_GBS, 4),
+                    "kernel_ms": round(stages["gate_up_gemm_act"], 4),
+                    "traffic": MEASURED_TRAFFIC_BYTES[a.workload]}
+        value, unit, metric = gbs, "GB/s", METRIC + " [decode-only workload: HBM GB/s]"
+
+    out = {
+        "metric": metric, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": a.workload, "tokens": main_layer.T, "hidden": shape.hidden,
+                   "experts": shape.experts, "intermediate": shape.intermediate,
+                   "top_k": shape.top_k, "block_size_m": main_layer.bm, "active_experts": n_active},
+        "layer_tflops": round(tflops, 2), "layer_frac_of_bf16_peak": round(tflops / PEAK_BF16_TFLOPS, 4),
+        "layer_algorithmic_gbs": round(gbs, 1),
+        "stage_ms": {k: round(v, 4) for k, v in stages.items()},
+        "roofline": roofline,
+    }
+
+    if compute_bound:
+        dec = Layer(moe, "decode_256", dev)
+        dms = time_steps(dec, max(a.steps, 50), max(a.warmup, 10))
+        dstages, dids = time_stages(dec, 20)
+        dact = dec.n_active(dids)
+        dbytes = wl.layer_bytes(dec.T, dec.shape, dact)
+        dgbs = dbytes / (dms * 1e-3) / 1e9
+        out["decode"] = {"workload": "decode_256", "tokens": dec.T, "ms_per_step": round(dms, 4),
+                         "hbm_gbs": round(dgbs, 1), "frac_of_hbm_peak": round(dgbs / PEAK_HBM_GBS, 4),
+                         "active_experts": dact, "block_size_m": dec.bm,
+                         "stage_ms": {k: round(v, 4) for k, v in dstages.items()}}
+        del dec
+
+    if not a.no_cpu_baseline:
+        del main_layer
+        torch.cuda.empty_cache()
+        dt, cores = cpu_baseline(moe, a.workload, a.cpu_runs)
+        if compute_bound:
+            cv, cu = flops / dt / 1e12, "TFLOP/s"
+        else:
+            cv, cu = abytes / dt / 1e9, "GB/s"
+        out["cpu_baseline"] = {"value": round(cv, 4), "unit": cu, "cores": cores, "kind": "port",
+                               "sample": f"{a.cpu_runs} full passes of {a.workload} (1 warm-up), "
+                                         f"oracle fp32 torch matmul, bf16 weights upcast per expert, "
+                                         f"{dt:.2f} s per pass"}
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

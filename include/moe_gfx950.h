@@ -117,6 +117,11 @@ typedef struct MoeFusedExpertsArgs {
   int32_t activation;        /* MoeActivation                                        */
   int32_t apply_router_weight_on_input;
   float swiglu_alpha, swiglu_limit;
+  /* bit mask of the passes to enqueue: 1 gate-up GEMM + activation, 2 down GEMM
+     times routed weight, 4 top-k combine; 0 means all three.  Lets a profiler
+     or benchmark time one pass alone (the later passes then read whatever the
+     workspace holds). */
+  int32_t passes;
   void* stream;
 } MoeFusedExpertsArgs;
 

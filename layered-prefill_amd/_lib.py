@@ -46,7 +46,7 @@ class MoeFusedExpertsArgs(ctypes.Structure):
         ("weight_dtype", ctypes.c_int32), ("activation", ctypes.c_int32),
         ("apply_router_weight_on_input", ctypes.c_int32),
         ("swiglu_alpha", ctypes.c_float), ("swiglu_limit", ctypes.c_float),
-        ("stream", ctypes.c_void_p),
+        ("passes", ctypes.c_int32), ("stream", ctypes.c_void_p),
     ]
 
 

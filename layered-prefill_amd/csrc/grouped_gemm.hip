@@ -383,8 +383,11 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.bias = a->w13_bias; p.bias_stride_e = 2LL * a->I;
   p.c = inter; p.ldc = a->I; p.Kd = a->H; p.N = a->I; p.a_by_slot = 0;
   p.mul_weight = a->apply_router_weight_on_input ? 1 : 0;
-  int rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaBF16, true>(p, a->block_size, a->sorted_cap, s)
-                                    : launch_bm<MmaF16, true>(p, a->block_size, a->sorted_cap, s);
+  const int passes = a->passes ? a->passes : 7;
+  int rc = MOE_OK;
+  if (passes & 1)
+    rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaBF16, true>(p, a->block_size, a->sorted_cap, s)
+                                  : launch_bm<MmaF16, true>(p, a->block_size, a->sorted_cap, s);
   if (rc) return rc;
 
   // pass 2: inter . W2^T times the routed weight, rows written by flat token id
@@ -392,10 +395,12 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.bias = a->w2_bias; p.bias_stride_e = a->H;
   p.c = c3; p.ldc = a->H; p.Kd = a->I; p.N = a->H; p.a_by_slot = 1;
   p.mul_weight = a->apply_router_weight_on_input ? 0 : 1;
-  rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaBF16, false>(p, a->block_size, a->sorted_cap, s)
-                                : launch_bm<MmaF16, false>(p, a->block_size, a->sorted_cap, s);
+  if (passes & 2)
+    rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaBF16, false>(p, a->block_size, a->sorted_cap, s)
+                                  : launch_bm<MmaF16, false>(p, a->block_size, a->sorted_cap, s);
   if (rc) return rc;
 
   // top-k combine (nanovllm/layers/for_moe/moe_easy_kernel.py:26-31)
+  if (!(passes & 4)) return MOE_OK;
   return moe_sum(a->out, c3, a->T, a->K, a->H, a->act_dtype, a->stream);
 }

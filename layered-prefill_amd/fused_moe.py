@@ -93,6 +93,63 @@ def fused_experts(hidden_states: torch.Tensor,
                               block_shape, w1_bias, w2_bias)
 
 
+def fused_experts_workspace_bytes(tokens: int, hidden: int, intermediate: int, experts: int,
+                                  top_k: int, block_size: int, act_dtype: torch.dtype,
+                                  weight_code: Optional[int] = None) -> int:
+    act_code = _lib.DTYPE_CODE[act_dtype]
+    return lib().moe_fused_experts_workspace_bytes(
+        tokens, hidden, intermediate, experts, top_k, block_size, act_code,
+        act_code if weight_code is None else weight_code)
+
+
+def launch_fused_experts(x: torch.Tensor, out: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
+                         w1_bias: Optional[torch.Tensor], w2_bias: Optional[torch.Tensor],
+                         w1_scale: Optional[torch.Tensor], w2_scale: Optional[torch.Tensor],
+                         topk_weights: torch.Tensor, sorted_token_ids: torch.Tensor,
+                         expert_ids: torch.Tensor, num_tokens_post_padded: torch.Tensor,
+                         block_size: int, activation: str = "silu",
+                         apply_router_weight_on_input: bool = False,
+                         weight_code: Optional[int] = None,
+                         workspace: Optional[torch.Tensor] = None, passes: int = 0) -> None:
+    """One call of the C entry point ``moe_fused_experts`` on already aligned
+    tokens (the part of nanovllm/layers/for_moe/fused_moe.py:579-631 after
+    moe_align_block_size).  ``workspace`` (uint8) is allocated when not given;
+    ``passes`` selects single passes for profiling (1 gate-up, 2 down, 4
+    combine, 0 = all)."""
+    T, H = x.shape
+    E, N, _ = w1.shape
+    top_k = topk_weights.shape[1]
+    act_code = _lib.DTYPE_CODE[x.dtype]
+    if weight_code is None:
+        weight_code = act_code
+    L = lib()
+    ws_bytes = L.moe_fused_experts_workspace_bytes(T, H, N // 2, E, top_k, block_size, act_code,
+                                                   weight_code)
+    if workspace is None:
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+    for name, b in (("w1_bias", w1_bias), ("w2_bias", w2_bias)):
+        if b is not None:
+            assert b.is_contiguous() and b.dtype == x.dtype, f"{name} must be contiguous {x.dtype}"
+    args = MoeFusedExpertsArgs(
+        x=x.data_ptr(), out=out.data_ptr(), w13=w1.data_ptr(), w2=w2.data_ptr(),
+        w13_bias=w1_bias.data_ptr() if w1_bias is not None else None,
+        w2_bias=w2_bias.data_ptr() if w2_bias is not None else None,
+        w13_scale=w1_scale.data_ptr() if w1_scale is not None else None,
+        w2_scale=w2_scale.data_ptr() if w2_scale is not None else None,
+        topk_weights=topk_weights.data_ptr(), sorted_token_ids=sorted_token_ids.data_ptr(),
+        expert_ids=expert_ids.data_ptr(), num_tokens_post_pad=num_tokens_post_padded.data_ptr(),
+        workspace=workspace.data_ptr(), workspace_bytes=workspace.numel(),
+        w13_stride_e=w1.stride(0), w13_stride_n=w1.stride(1),
+        w2_stride_e=w2.stride(0), w2_stride_n=w2.stride(1),
+        T=T, H=H, I=N // 2, E=E, K=top_k, block_size=block_size,
+        sorted_cap=sorted_token_ids.numel(), act_dtype=act_code, weight_dtype=weight_code,
+        activation=_lib.ACTIVATION_CODE[activation],
+        apply_router_weight_on_input=int(apply_router_weight_on_input),
+        swiglu_alpha=1.702, swiglu_limit=7.0, passes=passes, stream=stream_ptr(x.device))
+    with torch.cuda.device(x.device):
+        check(L.moe_fused_experts(args))
+
+
 _FP8_DTYPES = tuple(getattr(torch, n) for n in ("float8_e4m3fn",) if hasattr(torch, n))
 
 
@@ -178,30 +235,8 @@ def fused_experts_impl(hidden_states: torch.Tensor,
         curr_w = topk_weights[begin:end]
         sorted_token_ids, expert_ids, num_tokens_post_padded = moe_align_block_size(
             curr_ids, bm, global_num_experts)
-        ws_bytes = L.moe_fused_experts_workspace_bytes(tokens_in_chunk, K, N // 2, E, top_k_num, bm,
-                                                       act_code, weight_code)
-        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-        args = MoeFusedExpertsArgs(
-            x=hidden_states[begin:end].data_ptr(), out=out_hidden_states[begin:end].data_ptr(),
-            w13=w1.data_ptr(), w2=w2.data_ptr(),
-            w13_bias=w1_bias.data_ptr() if w1_bias is not None else None,
-            w2_bias=w2_bias.data_ptr() if w2_bias is not None else None,
-            w13_scale=w1_scale.data_ptr() if w1_scale is not None else None,
-            w2_scale=w2_scale.data_ptr() if w2_scale is not None else None,
-            topk_weights=curr_w.data_ptr(), sorted_token_ids=sorted_token_ids.data_ptr(),
-            expert_ids=expert_ids.data_ptr(), num_tokens_post_pad=num_tokens_post_padded.data_ptr(),
-            workspace=workspace.data_ptr(), workspace_bytes=ws_bytes,
-            w13_stride_e=w1.stride(0), w13_stride_n=w1.stride(1),
-            w2_stride_e=w2.stride(0), w2_stride_n=w2.stride(1),
-            T=tokens_in_chunk, H=K, I=N // 2, E=E, K=top_k_num, block_size=bm,
-            sorted_cap=sorted_token_ids.numel(), act_dtype=act_code, weight_dtype=weight_code,
-            activation=_lib.ACTIVATION_CODE[activation],
-            apply_router_weight_on_input=int(apply_router_weight_on_input),
-            swiglu_alpha=1.702, swiglu_limit=7.0, stream=stream_ptr(dev))
-        if w1_bias is not None:
-            assert w1_bias.is_contiguous() and w1_bias.dtype == hidden_states.dtype
-        if w2_bias is not None:
-            assert w2_bias.is_contiguous() and w2_bias.dtype == hidden_states.dtype
-        with torch.cuda.device(dev):
-            check(L.moe_fused_experts(args))
+        launch_fused_experts(hidden_states[begin:end], out_hidden_states[begin:end], w1, w2,
+                             w1_bias, w2_bias, w1_scale, w2_scale, curr_w, sorted_token_ids,
+                             expert_ids, num_tokens_post_padded, bm, activation,
+                             apply_router_weight_on_input, weight_code=weight_code)
     return out_hidden_states
