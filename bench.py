@@ -145,6 +145,8 @@ def main() -> int:
                     choices=["layered_8192p_256d", "decode_256"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-runs", type=int, default=2)
+    ap.add_argument("--block-size-m", type=int, default=0,
+                    help="override the alignment block size (0 = the library's choice)")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build is the single-GPU (TP=1) expert path; it has no collectives "
@@ -158,6 +160,9 @@ def main() -> int:
     dev = torch.device("cuda:0")
     wl = moe.workloads
 
+    if a.block_size_m:
+        moe.fused_moe.try_get_optimal_moe_config = lambda *x, **k: {"BLOCK_SIZE_M": a.block_size_m}
+        moe.try_get_optimal_moe_config = moe.fused_moe.try_get_optimal_moe_config
     main_layer = Layer(moe, a.workload, dev)
     ms = time_steps(main_layer, a.steps, a.warmup)
     stages, ids = time_stages(main_layer, max(5, a.steps // 2))

@@ -15,6 +15,8 @@
 // groups) and feed v_mfma_f32_32x32x16.  The weight fragment is the A operand
 // and the token fragment the B operand, so that a lane ends up with four
 // consecutive output columns of one token and stores them as one 8-byte word.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace {
@@ -60,6 +62,7 @@ struct GemmParams {
   int activation;    // MoeActivation (gated pass only)
   int interleaved;   // gate/up rows interleaved (2n, 2n+1) instead of halves (n, N+n)
   float alpha, limit;
+  int m_major;       // workgroup order inside an XCD: all n-tiles of an m-block are neighbours
 };
 
 constexpr int kThreads = 256;
@@ -71,10 +74,68 @@ __device__ __forceinline__ int swizzled(int row, int chunk) {
   return row * kRowBytes + ((chunk ^ ((row >> 1) & 7)) << 4);
 }
 
+
+// Writes one 32x32 accumulator fragment (pair, when gated): this lane holds, for
+// token `tok` (slot `slot`), the output columns ncol0 + 8*g + i, g,i in 0..3.
+// Rounding follows the reference's storage points: the GEMM result is rounded to
+// the activation dtype, silu is rounded, the product is rounded
+// (nanovllm/layers/for_moe/fused_moe.py:216, csrc/activation_kernels.cu:11,23).
+template <typename El, bool GATED>
+__device__ __forceinline__ void store_fragment(const GemmParams& p, int e, const f32x16& ga,
+                                               const f32x16& ua, int tok, int slot, int ncol0) {
+  using S = typename El::S;
+  const S* bias = static_cast<const S*>(p.bias);
+  const float rw = p.mul_weight ? p.topk_w[tok] : 1.f;
+  const int64_t crow = p.a_by_slot ? tok : slot;  // pass 2 writes by token, pass 1 by slot
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int n = ncol0 + 8 * g;
+    S o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int col = (n + i < p.N) ? n + i : p.N - 1;
+      if constexpr (GATED) {
+        float gv = ga[4 * g + i], uv = ua[4 * g + i];
+        if (bias) {
+          const int64_t grow = p.interleaved ? 2 * col : col;
+          const int64_t urow = p.interleaved ? 2 * col + 1 : p.N + col;
+          gv += El::ld(bias[e * p.bias_stride_e + grow]);
+          uv += El::ld(bias[e * p.bias_stride_e + urow]);
+        }
+        if (p.mul_weight) { gv *= rw; uv *= rw; }
+        gv = El::ld(El::st(gv));
+        uv = El::ld(El::st(uv));
+        float r;
+        if (p.activation == MOE_ACT_SILU) {
+          r = El::ld(El::st(moe_silu(gv))) * uv;
+        } else if (p.activation == MOE_ACT_SWIGLUOAI) {
+          r = moe_swigluoai(gv, uv, p.alpha, p.limit);
+        } else {
+          const float ge = 0.5f * gv * (1.f + erff(gv * 0.70710678118654752f));
+          r = El::ld(El::st(ge)) * uv;
+        }
+        o[i] = El::st(r);
+      } else {
+        float v = ga[4 * g + i];
+        if (bias) v += El::ld(bias[e * p.bias_stride_e + col]);
+        o[i] = El::st(v * rw);
+      }
+    }
+    S* dst = static_cast<S*>(p.c) + crow * p.ldc + n;
+    if (n + 3 < p.N && (p.ldc & 3) == 0) {
+      *reinterpret_cast<uint2*>(dst) = uint2{static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16),
+                                             static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16)};
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n + i < p.N) dst[i] = o[i];
+    }
+  }
+}
+
 template <typename Mma, int BM, int BNW, int WAVES_M, bool GATED>
 __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams p) {
   using El = typename Mma::El;
-  using S = typename El::S;
   constexpr int WAVES_N = 4 / WAVES_M;
   constexpr int TM = BM / WAVES_M, FM = TM / 32;     // token fragments per wavefront
   constexpr int TNW = BNW / WAVES_N, FN = TNW / 32;  // weight-row fragments per wavefront
@@ -91,8 +152,14 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
   const int per_xcd = gridDim.x / kXcds;
   const int logical = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
   if (logical >= p.num_m_blocks * p.num_n_tiles) return;
-  const int nt = logical / p.num_m_blocks;
-  const int mb = logical - nt * p.num_m_blocks;
+  int nt, mb;
+  if (p.m_major) {
+    mb = logical / p.num_n_tiles;
+    nt = logical - mb * p.num_n_tiles;
+  } else {
+    nt = logical / p.num_m_blocks;
+    mb = logical - nt * p.num_m_blocks;
+  }
   if (mb * BM >= *p.num_post_pad) return;
   const int e = p.expert_ids[mb];
   const int n0 = nt * BN_OUT;
@@ -203,64 +270,583 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
 
   // Epilogue.  acc[fn][fm][r]: weight row 8*(r/4) + 4*(lane/32) + r%4 of
   // fragment fn, token row lane%32 of fragment fm.
-  S* cbase = static_cast<S*>(p.c);
-  const S* bias = static_cast<const S*>(p.bias);
 #pragma unroll
   for (int fm = 0; fm < FM; ++fm) {
     const int slot = mb * BM + wm * TM + fm * 32 + l32;
     const int tok = p.sorted_ids[slot];
     if (tok >= p.numel) continue;  // padding slot
-    const float rw = p.mul_weight ? p.topk_w[tok] : 1.f;
-    const int64_t crow = p.a_by_slot ? tok : slot;  // pass 2 writes by token, pass 1 by slot
 #pragma unroll
     for (int fo = 0; fo < FNO; ++fo) {
       const int ncol0 = n0 + (GATED ? wn * (TNW / 2) : wn * TNW) + fo * 32 + 4 * lhi;
+      store_fragment<El, GATED>(p, e, acc[fo][fm], acc[GATED ? fo + FNO : fo][fm], tok, slot, ncol0);
+    }
+  }
+}
+
+
+// ---------------------------------------------------------------------------
+// Weight-streaming variant.  The token tile (BM = 32*FM rows) is shared by the
+// four wavefronts through LDS; every wavefront owns 64 weight rows of the strip
+// (32 gate + 32 up rows of the same output columns when gated) and loads them
+// from global memory straight into registers, 64 contiguous bytes per lane and
+// K tile, WDEPTH K tiles ahead.  Weights therefore never pass through LDS, and
+// one token fragment read from LDS feeds two MFMAs.  Lane (r, h) of a weight
+// fragment holds K elements [32h, 32h+32) of the 64-wide K tile, so MFMA step j
+// multiplies 16-byte chunk 4h+j of both operands (any pairing of K elements is
+// a valid dot product as long as both operands use the same one).
+// Token fragments that hold only padding slots are skipped.
+// ---------------------------------------------------------------------------
+template <typename Mma, int FM, int WDEPTH, bool GATED>
+__global__ __launch_bounds__(kThreads) void wstream_gemm_kernel(const GemmParams p) {
+  using El = typename Mma::El;
+  constexpr int BM = FM * 32;
+  constexpr int NOUT_WAVE = GATED ? 32 : 64;  // output columns per wavefront
+  constexpr int BN_OUT = 4 * NOUT_WAVE;
+  constexpr int STAGE_BYTES = BM * kRowBytes;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int per_xcd = gridDim.x / kXcds;
+  const int logical = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
+  if (logical >= p.num_m_blocks * p.num_n_tiles) return;
+  int nt, mb;
+  if (p.m_major) {
+    mb = logical / p.num_n_tiles;
+    nt = logical - mb * p.num_n_tiles;
+  } else {
+    nt = logical / p.num_m_blocks;
+    mb = logical - nt * p.num_m_blocks;
+  }
+  if (mb * BM >= *p.num_post_pad) return;
+  const int e = p.expert_ids[mb];
+  const int n0 = nt * BN_OUT;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, lhi = lane >> 5;
+  const int ld_row = tid >> 3, ld_c = tid & 7;
+
+  // real slots come first in a block: count them, whole fragments past them are skipped
+  int my_tok = p.numel;
+  if (tid < BM) my_tok = p.sorted_ids[mb * BM + tid];
+  const int nvalid = __syncthreads_count(my_tok < p.numel);
+  const int fm_eff = (nvalid + 31) >> 5;
+  if (fm_eff == 0) return;
+
+  const char* a_src[FM];
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int n = ncol0 + 8 * g;
-        S o[4];
+  for (int j = 0; j < FM; ++j) {
+    const int slot = mb * BM + ld_row + 32 * j;
+    int64_t src = slot;
+    if (!p.a_by_slot) {
+      const int tok = p.sorted_ids[slot];
+      src = tok < p.numel ? tok / p.top_k : 0;
+    }
+    a_src[j] = static_cast<const char*>(p.a) + (src * p.lda + ld_c * 8) * 2;
+  }
+  const char* w_src[2];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int col = (n + i < p.N) ? n + i : p.N - 1;
-          if constexpr (GATED) {
-            float gv = acc[fo][fm][4 * g + i], uv = acc[fo + FNO][fm][4 * g + i];
-            if (bias) {
-              const int64_t grow = p.interleaved ? 2 * col : col;
-              const int64_t urow = p.interleaved ? 2 * col + 1 : p.N + col;
-              gv += El::ld(bias[e * p.bias_stride_e + grow]);
-              uv += El::ld(bias[e * p.bias_stride_e + urow]);
+  for (int f = 0; f < 2; ++f) {
+    int64_t wrow;
+    if constexpr (GATED) {
+      int n = n0 + wave * 32 + l32;
+      n = n < p.N ? n : p.N - 1;
+      wrow = p.interleaved ? (2 * n + f) : (f * p.N + n);
+    } else {
+      const int n = n0 + wave * 64 + f * 32 + l32;
+      wrow = n < p.N ? n : p.N - 1;
+    }
+    w_src[f] = static_cast<const char*>(p.w) +
+               (static_cast<int64_t>(e) * p.w_stride_e + wrow * p.w_stride_n + lhi * 32) * 2;
+  }
+  const int st_off = swizzled(ld_row, ld_c);
+  int rd_k[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) rd_k[j] = l32 * kRowBytes + (((4 * lhi + j) ^ ((l32 >> 1) & 7)) << 4);
+
+  f32x16 acc[2][FM];
+#pragma unroll
+  for (int f = 0; f < 2; ++f)
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[f][fm][r] = 0.f;
+
+  uint4 t_reg[FM];
+  uint4 w_reg[WDEPTH][2][4];
+  const int nk = (p.Kd + kBK - 1) / kBK;
+  const bool k_exact = (p.Kd % kBK) == 0;
+
+  auto load_tokens = [&](int kt) {
+    const bool in_k = k_exact || kt * kBK + ld_c * 8 < p.Kd;
+#pragma unroll
+    for (int j = 0; j < FM; ++j)
+      if (j < fm_eff)
+        t_reg[j] = in_k ? *reinterpret_cast<const uint4*>(a_src[j] + kt * kRowBytes) : uint4{0, 0, 0, 0};
+  };
+  auto store_tokens = [&](int stage) {
+    char* base = smem + stage * STAGE_BYTES + st_off;
+#pragma unroll
+    for (int j = 0; j < FM; ++j)
+      if (j < fm_eff) *reinterpret_cast<uint4*>(base + j * 32 * kRowBytes) = t_reg[j];
+  };
+  auto load_weights = [&](int kt, uint4 (&dst)[2][4]) {
+#pragma unroll
+    for (int f = 0; f < 2; ++f)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bool in_k = k_exact || kt * kBK + lhi * 32 + j * 8 < p.Kd;
+        dst[f][j] = in_k ? *reinterpret_cast<const uint4*>(w_src[f] + kt * kRowBytes + j * 16)
+                         : uint4{0, 0, 0, 0};
+      }
+  };
+
+  // prologue: weights for tiles 0 .. WDEPTH-2, tokens for tile 0
+#pragma unroll
+  for (int d = 0; d < WDEPTH - 1; ++d)
+    if (d < nk) load_weights(d, w_reg[d]);
+  load_tokens(0);
+  store_tokens(0);
+  __syncthreads();
+
+  for (int kt0 = 0; kt0 < nk; kt0 += WDEPTH) {
+#pragma unroll
+    for (int d = 0; d < WDEPTH; ++d) {
+      const int kt = kt0 + d;
+      if (kt < nk) {
+        if (kt + WDEPTH - 1 < nk) load_weights(kt + WDEPTH - 1, w_reg[(d + WDEPTH - 1) % WDEPTH]);
+        if (kt + 1 < nk) load_tokens(kt + 1);
+        const char* st = smem + (kt & 1) * STAGE_BYTES;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+          for (int fm = 0; fm < FM; ++fm) {
+            if (fm < fm_eff) {
+              const uint4 xf = *reinterpret_cast<const uint4*>(st + fm * 32 * kRowBytes + rd_k[j]);
+              acc[0][fm] = Mma::mma(w_reg[d][0][j], xf, acc[0][fm]);
+              acc[1][fm] = Mma::mma(w_reg[d][1][j], xf, acc[1][fm]);
             }
-            if (p.mul_weight) { gv *= rw; uv *= rw; }
-            gv = El::ld(El::st(gv));  // the reference stores GEMM1's result in T
-            uv = El::ld(El::st(uv));
-            float r;
-            if (p.activation == MOE_ACT_SILU) {
-              r = El::ld(El::st(moe_silu(gv))) * uv;
-            } else if (p.activation == MOE_ACT_SWIGLUOAI) {
-              r = moe_swigluoai(gv, uv, p.alpha, p.limit);
-            } else {
-              const float ge = 0.5f * gv * (1.f + erff(gv * 0.70710678118654752f));
-              r = El::ld(El::st(ge)) * uv;
-            }
-            o[i] = El::st(r);
-          } else {
-            float v = acc[fo][fm][4 * g + i];
-            if (bias) v += El::ld(bias[e * p.bias_stride_e + col]);
-            o[i] = El::st(v * rw);
           }
         }
-        S* dst = cbase + crow * p.ldc + n;
-        if (n + 3 < p.N && (p.ldc & 3) == 0) {
-          *reinterpret_cast<uint2*>(dst) = uint2{static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16),
-                                                 static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16)};
-        } else {
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (n + i < p.N) dst[i] = o[i];
-        }
+        if (kt + 1 < nk) store_tokens((kt + 1) & 1);
+        __syncthreads();
       }
     }
   }
+
+#pragma unroll
+  for (int fm = 0; fm < FM; ++fm) {
+    if (fm >= fm_eff) continue;
+    const int slot = mb * BM + fm * 32 + l32;
+    const int tok = p.sorted_ids[slot];
+    if (tok >= p.numel) continue;
+    if constexpr (GATED) {
+      store_fragment<El, true>(p, e, acc[0][fm], acc[1][fm], tok, slot, n0 + wave * 32 + 4 * lhi);
+    } else {
+      store_fragment<El, false>(p, e, acc[0][fm], acc[0][fm], tok, slot, n0 + wave * 64 + 4 * lhi);
+      store_fragment<El, false>(p, e, acc[1][fm], acc[1][fm], tok, slot, n0 + wave * 64 + 32 + 4 * lhi);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Large-tile variant for compute-bound calls: 256 slots x 256 weight rows per
+// workgroup, one wavefront per SIMD, each owning a 128 x 128 register tile
+// (16 accumulator fragments in AGPRs), so one 16-byte fragment read from LDS
+// feeds four MFMAs.  K advances in 32-element tiles through a 4-stage LDS ring
+// filled by direct global->LDS loads (global_load_lds_dwordx4): three tiles are
+// in flight while one is consumed, and the only per-tile synchronisation is one
+// vmcnt wait plus one s_barrier.  The loads are issued from inline assembly so
+// that the vmcnt bookkeeping is exactly the one written here.
+// Staged rows are 64 bytes; 16-byte chunk c of row r sits at chunk
+// c ^ ((r >> 2) & 3), which makes both the DMA writes (4 lanes per row) and the
+// fragment reads (16 consecutive rows, one chunk) touch 16 distinct 16-byte
+// bank groups.  Token fragments holding only padding slots are skipped.
+// The epilogue rounds the accumulators to the activation dtype, parks the
+// wavefront's 128 x 128 tile in LDS and writes it out with 16-byte stores, the
+// gated activation being applied on the way.
+// ---------------------------------------------------------------------------
+constexpr int kBigBM = 256, kBigBNW = 256, kBigBK = 32, kBigStages = 4;
+constexpr int kBigRowBytes = kBigBK * 2;
+constexpr int kBigStageBytes = (kBigBM + kBigBNW) * kBigRowBytes;
+constexpr int kBigDmaPerTile = 8;            // global_load_lds instructions per thread and K tile
+constexpr int kEpiRowBytes = 128 * 2 + 16;   // one token row of a wavefront's tile, padded
+constexpr int kEpiWaveBytes = 128 * kEpiRowBytes;
+constexpr int kBigLdsBytes = 4 * kEpiWaveBytes > kBigStages * kBigStageBytes ? 4 * kEpiWaveBytes
+                                                                              : kBigStages * kBigStageBytes;
+
+typedef __attribute__((address_space(3))) char lds_char;
+
+__device__ __forceinline__ uint32_t lds_offset_of(const char* p) {
+  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const lds_char*)p));
+}
+
+// 16 bytes per lane from global memory straight into LDS at
+// lds_wave_base + 16 * lane.  `base` and `lds_wave_base` are wavefront-uniform.
+__device__ __forceinline__ void lds_dma16(const char* base, uint32_t lane_byte_offset,
+                                          uint32_t lds_wave_base) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2"
+      :
+      : "s"(lds_wave_base), "v"(lane_byte_offset), "s"(base)
+      : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ void bare_barrier() {
+  asm volatile("s_barrier" ::: "memory");
+}
+
+template <typename El>
+__device__ __forceinline__ uint32_t pack2(float a, float b);
+template <>
+__device__ __forceinline__ uint32_t pack2<ElemBF16>(float a, float b) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2;
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+}
+template <>
+__device__ __forceinline__ uint32_t pack2<ElemF16>(float a, float b) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2;
+  typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, f16x2));
+}
+
+struct BigCtx {
+  const char* a_base;   // wave-uniform base of the A rows
+  const char* w_base;   // wave-uniform base of this expert's weights
+  uint32_t a_off[4];    // per-lane byte offsets of the four 64-row load groups
+  uint32_t w_off[4];
+  uint32_t dma_lds;     // LDS offset of this wavefront's DMA window in stage 0, group 0
+  int rd_k[2];          // fragment read offsets for the two MFMA steps of a K tile
+  int x_row;            // byte offset of this wavefront's first token row in a stage
+  int w_row[4];         // byte offsets of this wavefront's weight fragments in a stage
+};
+
+// Main loop for a wavefront that has FMC live token fragments (0..4).
+// Schedule of one K tile (two MFMA steps, fragment sets P and Q in registers):
+//   read Q <- (kt, step 1) | 16 MFMAs on P | wait tile kt+1, barrier, issue tile
+//   kt+3 | read P <- (kt+1, step 0) | 16 MFMAs on Q
+// so the LDS reads of a step are always in flight behind the MFMAs of the
+// previous one.  sched_barrier keeps the compiler from re-serialising them.
+template <typename Mma, int FMC>
+__device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, int nk,
+                                             f32x16 (&acc)[4][4]) {
+  auto issue_tile = [&](int kt) {
+    const uint32_t dst = c.dma_lds + (kt % kBigStages) * kBigStageBytes;
+    const char* ab = c.a_base + kt * kBigRowBytes;
+    const char* wb = c.w_base + kt * kBigRowBytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) lds_dma16(ab, c.a_off[i], dst + i * 4096);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) lds_dma16(wb, c.w_off[i], dst + (4 + i) * 4096);
+  };
+  constexpr int XF = FMC > 0 ? FMC : 1;
+  auto read_frags = [&](int kt, int kk, uint4 (&wf)[4], uint4 (&xf)[XF]) {
+    if constexpr (FMC > 0) {
+      const char* st = smem + (kt % kBigStages) * kBigStageBytes;
+#pragma unroll
+      for (int fn = 0; fn < 4; ++fn) wf[fn] = *reinterpret_cast<const uint4*>(st + c.w_row[fn] + c.rd_k[kk]);
+#pragma unroll
+      for (int fm = 0; fm < FMC; ++fm)
+        xf[fm] = *reinterpret_cast<const uint4*>(st + c.x_row + fm * 32 * kBigRowBytes + c.rd_k[kk]);
+    }
+  };
+  auto mma_all = [&](const uint4 (&wf)[4], const uint4 (&xf)[XF]) {
+#pragma unroll
+    for (int fm = 0; fm < FMC; ++fm)
+#pragma unroll
+      for (int fn = 0; fn < 4; ++fn) acc[fn][fm] = Mma::mma(wf[fn], xf[fm], acc[fn][fm]);
+  };
+
+  // tiles 0..2 in flight, tile 0 landed and visible, fragments of (0, step 0) requested
+  issue_tile(0);
+  if (1 < nk) issue_tile(1);
+  if (2 < nk) issue_tile(2);
+  if (2 < nk) wait_vmcnt<2 * kBigDmaPerTile>();
+  else if (1 < nk) wait_vmcnt<kBigDmaPerTile>();
+  else wait_vmcnt<0>();
+  bare_barrier();
+  uint4 wfP[4], xfP[XF], wfQ[4], xfQ[XF];
+  read_frags(0, 0, wfP, xfP);
+  __builtin_amdgcn_sched_barrier(0);
+
+  for (int kt = 0; kt < nk; ++kt) {
+    read_frags(kt, 1, wfQ, xfQ);
+    __builtin_amdgcn_sched_barrier(0);
+    mma_all(wfP, xfP);
+    __builtin_amdgcn_sched_barrier(0);
+    if (kt + 1 < nk) {
+      // tile kt+1 must have landed; tile kt+2 may still be in flight
+      if (kt + 2 < nk) wait_vmcnt<kBigDmaPerTile>();
+      else wait_vmcnt<0>();
+      bare_barrier();
+      if (kt + 3 < nk) issue_tile(kt + 3);  // into the stage of tile kt-1, fully consumed
+      read_frags(kt + 1, 0, wfP, xfP);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    mma_all(wfQ, xfQ);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// Epilogue phase 1: round this wavefront's accumulators to the activation dtype
+// (after the optional bias and routed weight) and park them in its LDS window
+// as [token row][weight row].
+template <typename El, int FMC, bool GATED>
+__device__ __forceinline__ void big_park(const GemmParams& p, int e, int n0, int wn, int lhi, int l32,
+                                         int slot0, char* epi, const f32x16 (&acc)[4][4]) {
+  using S = typename El::S;
+  const S* bias = static_cast<const S*>(p.bias);
+#pragma unroll
+  for (int fm = 0; fm < FMC; ++fm) {
+    float rw = 1.f;
+    if (p.mul_weight) {
+      const int tok = p.sorted_ids[slot0 + fm * 32 + l32];
+      rw = tok < p.numel ? p.topk_w[tok] : 0.f;
+    }
+    char* row = epi + (fm * 32 + l32) * kEpiRowBytes;
+#pragma unroll
+    for (int fn = 0; fn < 4; ++fn) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = acc[fn][fm][4 * g + i];
+        if (bias) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int local = fn * 32 + 8 * g + 4 * lhi + i;  // column inside the wavefront tile
+            int64_t brow;
+            if constexpr (GATED) {
+              int col = n0 + wn * 64 + (local & 63);
+              col = col < p.N ? col : p.N - 1;
+              const int half = local >> 6;
+              brow = p.interleaved ? 2 * col + half : half * p.N + col;
+            } else {
+              const int col = n0 + wn * 128 + local;
+              brow = col < p.N ? col : p.N - 1;
+            }
+            v[i] += El::ld(bias[e * p.bias_stride_e + brow]);
+          }
+        }
+        if (p.mul_weight) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] *= rw;
+        }
+        *reinterpret_cast<uint2*>(row + (fn * 32 + 8 * g + 4 * lhi) * 2) =
+            uint2{pack2<El>(v[0], v[1]), pack2<El>(v[2], v[3])};
+      }
+    }
+  }
+}
+
+// Epilogue phase 2: write the parked tile to global memory, 8 columns (16 bytes)
+// per lane and step.  Gated: columns [0,64) of a row are gate values, [64,128)
+// the matching up values.
+template <typename El, bool GATED>
+__device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, int lane, int slot0,
+                                          int rows, const char* epi) {
+  using S = typename El::S;
+  constexpr int COLS = GATED ? 64 : 128;      // output columns of the wavefront tile
+  constexpr int LPR = COLS / 8;               // lanes per row
+  constexpr int RPS = kWave / LPR;            // rows per step
+  const int c8 = (lane % LPR) * 8;
+  const int ncol = n0 + wn * COLS + c8;
+  for (int r0 = 0; r0 < rows; r0 += RPS) {
+    const int r = r0 + lane / LPR;
+    if (r >= rows) continue;
+    const int slot = slot0 + r;
+    const int tok = p.sorted_ids[slot];
+    if (tok >= p.numel) continue;
+    const char* row = epi + r * kEpiRowBytes;
+    uint4 out;
+    if constexpr (GATED) {
+      const uint4 gq = *reinterpret_cast<const uint4*>(row + c8 * 2);
+      const uint4 uq = *reinterpret_cast<const uint4*>(row + (64 + c8) * 2);
+      const uint32_t gw[4] = {gq.x, gq.y, gq.z, gq.w}, uw[4] = {uq.x, uq.y, uq.z, uq.w};
+      uint32_t ow[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float res[2];
+#pragma unroll
+        for (int hlf = 0; hlf < 2; ++hlf) {
+          const float gv = El::ld(static_cast<S>(gw[i] >> (16 * hlf)));
+          const float uv = El::ld(static_cast<S>(uw[i] >> (16 * hlf)));
+          float rr;
+          if (p.activation == MOE_ACT_SILU) {
+            rr = El::ld(El::st(moe_silu(gv))) * uv;
+          } else if (p.activation == MOE_ACT_SWIGLUOAI) {
+            rr = moe_swigluoai(gv, uv, p.alpha, p.limit);
+          } else {
+            const float ge = 0.5f * gv * (1.f + erff(gv * 0.70710678118654752f));
+            rr = El::ld(El::st(ge)) * uv;
+          }
+          res[hlf] = rr;
+        }
+        ow[i] = static_cast<uint32_t>(El::st(res[0])) | (static_cast<uint32_t>(El::st(res[1])) << 16);
+      }
+      out = uint4{ow[0], ow[1], ow[2], ow[3]};
+    } else {
+      out = *reinterpret_cast<const uint4*>(row + c8 * 2);
+    }
+    const int64_t crow = p.a_by_slot ? tok : slot;
+    S* dst = static_cast<S*>(p.c) + crow * p.ldc + ncol;
+    if (ncol + 7 < p.N && (p.ldc & 7) == 0) {
+      *reinterpret_cast<uint4*>(dst) = out;
+    } else {
+      const uint32_t w4[4] = {out.x, out.y, out.z, out.w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (ncol + i < p.N) dst[i] = static_cast<S>(w4[i >> 1] >> (16 * (i & 1)));
+    }
+  }
+}
+
+template <typename Mma, int FMC, bool GATED>
+__device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, char* smem, int nk,
+                                         int e, int n0, int wn, int lane, int slot0, char* epi) {
+  using El = typename Mma::El;
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int fn = 0; fn < 4; ++fn)
+#pragma unroll
+    for (int fm = 0; fm < 4; ++fm)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[fn][fm][r] = 0.f;
+  big_mainloop<Mma, FMC>(c, smem, nk, acc);
+  bare_barrier();  // every wavefront is done reading the stages before they are reused
+  if constexpr (FMC > 0) big_park<El, FMC, GATED>(p, e, n0, wn, lane >> 5, lane & 31, slot0, epi, acc);
+}
+
+template <typename Mma, bool GATED>
+__global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams p) {
+  using El = typename Mma::El;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int per_xcd = gridDim.x / kXcds;
+  const int logical = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
+  if (logical >= p.num_m_blocks * p.num_n_tiles) return;
+  int nt, mb;
+  if (p.m_major) {
+    mb = logical / p.num_n_tiles;
+    nt = logical - mb * p.num_n_tiles;
+  } else {
+    nt = logical / p.num_m_blocks;
+    mb = logical - nt * p.num_m_blocks;
+  }
+  if (mb * kBigBM >= *p.num_post_pad) return;
+  const int e = p.expert_ids[mb];
+  const int n0 = nt * (GATED ? kBigBNW / 2 : kBigBNW);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, lhi = lane >> 5;
+  const int wm = wave & 1, wn = wave >> 1;
+  // real slots come first in a block
+  const int my_tok = p.sorted_ids[mb * kBigBM + tid];
+  const int nvalid = __syncthreads_count(my_tok < p.numel);
+  if (nvalid == 0) return;
+
+  BigCtx c;
+  const int ld_row = tid >> 2;                        // row inside a 64-row load group
+  const int ld_chunk = (tid & 3) ^ ((tid >> 4) & 3);  // logical chunk this lane fetches
+  c.a_base = static_cast<const char*>(p.a);
+  c.w_base = static_cast<const char*>(p.w) + static_cast<int64_t>(e) * p.w_stride_e * 2;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int slot = mb * kBigBM + ld_row + 64 * i;
+    int64_t src = slot;
+    if (!p.a_by_slot) {
+      const int tok = p.sorted_ids[slot];
+      src = tok < p.numel ? tok / p.top_k : 0;
+    }
+    c.a_off[i] = static_cast<uint32_t>((src * p.lda + ld_chunk * 8) * 2);
+    const int rr = ld_row + 64 * i;
+    int64_t wrow;
+    if constexpr (GATED) {
+      const int half = rr >> 7;
+      int n = n0 + (rr & 127);
+      n = n < p.N ? n : p.N - 1;
+      wrow = p.interleaved ? (2 * n + half) : (half * p.N + n);
+    } else {
+      const int n = n0 + rr;
+      wrow = n < p.N ? n : p.N - 1;
+    }
+    c.w_off[i] = static_cast<uint32_t>((wrow * p.w_stride_n + ld_chunk * 8) * 2);
+  }
+  c.dma_lds = __builtin_amdgcn_readfirstlane(lds_offset_of(smem) + wave * 1024);
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) c.rd_k[kk] = l32 * kBigRowBytes + (((2 * kk + lhi) ^ ((l32 >> 2) & 3)) << 4);
+  c.x_row = wm * 128 * kBigRowBytes;
+#pragma unroll
+  for (int fn = 0; fn < 4; ++fn) {
+    int r;
+    if constexpr (GATED)
+      r = (fn < 2) ? wn * 64 + fn * 32 : 128 + wn * 64 + (fn - 2) * 32;
+    else
+      r = wn * 128 + fn * 32;
+    c.w_row[fn] = (kBigBM + r) * kBigRowBytes;
+  }
+  const int nk = p.Kd / kBigBK;
+  const int slot0 = mb * kBigBM + wm * 128;
+  char* epi = smem + wave * kEpiWaveBytes;
+  const int rows = min(128, max(0, nvalid - wm * 128));  // real slots of this wavefront
+  switch ((rows + 31) >> 5) {
+    case 0: big_wave<Mma, 0, GATED>(p, c, smem, nk, e, n0, wn, lane, slot0, epi); break;
+    case 1: big_wave<Mma, 1, GATED>(p, c, smem, nk, e, n0, wn, lane, slot0, epi); break;
+    case 2: big_wave<Mma, 2, GATED>(p, c, smem, nk, e, n0, wn, lane, slot0, epi); break;
+    case 3: big_wave<Mma, 3, GATED>(p, c, smem, nk, e, n0, wn, lane, slot0, epi); break;
+    default: big_wave<Mma, 4, GATED>(p, c, smem, nk, e, n0, wn, lane, slot0, epi); break;
+  }
+  big_flush<El, GATED>(p, n0, wn, lane, slot0, rows, epi);
+}
+
+template <typename Mma, bool GATED>
+int launch_big(GemmParams& p, int64_t sorted_cap, hipStream_t s) {
+  constexpr int lds = kBigLdsBytes;
+  auto kern = big_gemm_kernel<Mma, GATED>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess)
+      return moe_fail(MOE_ERR_LAUNCH, "fused_experts: cannot reserve %d B of LDS: %s", lds, hipGetErrorString(e));
+    attr_set = true;
+  }
+  p.num_m_blocks = static_cast<int>((sorted_cap + kBigBM - 1) / kBigBM);
+  p.num_n_tiles = (p.N + (GATED ? 128 : 256) - 1) / (GATED ? 128 : 256);
+  const int64_t tiles = static_cast<int64_t>(p.num_m_blocks) * p.num_n_tiles;
+  const int64_t grid = (tiles + kXcds - 1) / kXcds * kXcds;
+  if (grid > INT32_MAX) return moe_fail(MOE_ERR_ARG, "fused_experts: grid of %lld workgroups", static_cast<long long>(grid));
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(kThreads), lds, s, p);
+  return moe_check_launch(GATED ? "fused_experts (gate-up pass)" : "fused_experts (down pass)");
+}
+
+template <typename Mma, int FM, int WDEPTH, bool GATED>
+int launch_wstream(GemmParams& p, int64_t sorted_cap, hipStream_t s) {
+  constexpr int BM = FM * 32;
+  constexpr int lds = 2 * BM * kRowBytes;
+  constexpr int bn_out = GATED ? 128 : 256;
+  p.num_m_blocks = static_cast<int>((sorted_cap + BM - 1) / BM);
+  p.num_n_tiles = (p.N + bn_out - 1) / bn_out;
+  auto kern = wstream_gemm_kernel<Mma, FM, WDEPTH, GATED>;
+  const int64_t tiles = static_cast<int64_t>(p.num_m_blocks) * p.num_n_tiles;
+  const int64_t grid = (tiles + kXcds - 1) / kXcds * kXcds;
+  if (grid > INT32_MAX) return moe_fail(MOE_ERR_ARG, "fused_experts: grid of %lld workgroups", static_cast<long long>(grid));
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(kThreads), lds, s, p);
+  return moe_check_launch(GATED ? "fused_experts (gate-up pass)" : "fused_experts (down pass)");
+}
+
+int gemm_variant() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("MOE_GEMM_VARIANT");
+    v = e ? atoi(e) : 0;
+  }
+  return v;
 }
 
 template <typename Mma, int BM, int BNW, int WAVES_M, bool GATED>
@@ -284,6 +870,17 @@ int launch(const GemmParams& p, hipStream_t s) {
 
 template <typename Mma, bool GATED>
 int launch_bm(GemmParams& p, int block_size, int64_t sorted_cap, hipStream_t s) {
+  if (block_size == 256 && p.Kd % kBigBK == 0 && gemm_variant() != 2) return launch_big<Mma, GATED>(p, sorted_cap, s);
+  if (gemm_variant() == 2) {
+    switch (block_size) {
+      case 256: return launch_wstream<Mma, 8, 2, GATED>(p, sorted_cap, s);
+      case 128: return launch_wstream<Mma, 4, 2, GATED>(p, sorted_cap, s);
+      case 64: return launch_wstream<Mma, 2, 3, GATED>(p, sorted_cap, s);
+      case 32: return launch_wstream<Mma, 1, 4, GATED>(p, sorted_cap, s);
+      default:
+        return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: block_size %d (supported: 32, 64, 128, 256)", block_size);
+    }
+  }
   p.num_m_blocks = static_cast<int>((sorted_cap + block_size - 1) / block_size);
   switch (block_size) {
     case 128:
@@ -377,6 +974,7 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.limit = a->swiglu_limit;
   p.activation = a->activation;
   p.interleaved = a->activation == MOE_ACT_SWIGLUOAI;
+  p.m_major = getenv("MOE_MAP") ? atoi(getenv("MOE_MAP")) : 0;
 
   // pass 1: x . W13^T with the gated activation, rows addressed by slot
   p.a = a->x; p.lda = a->H; p.w = a->w13; p.w_stride_e = a->w13_stride_e; p.w_stride_n = a->w13_stride_n;
