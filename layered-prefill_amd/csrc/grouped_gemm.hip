@@ -19,6 +19,14 @@
 
 #include "common.h"
 
+#ifdef MOE_TRACE
+// Development aid (make EXTRA=-DMOE_TRACE): per-workgroup phase timestamps of the large-tile kernel.
+__device__ unsigned long long moe_dbg[8 * 4096];
+#define MOE_TRACE_NOW() __builtin_amdgcn_s_memrealtime()
+#else
+#define MOE_TRACE_NOW() 0ull
+#endif
+
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -62,6 +70,7 @@ struct GemmParams {
   int activation;    // MoeActivation (gated pass only)
   int interleaved;   // gate/up rows interleaved (2n, 2n+1) instead of halves (n, N+n)
   float alpha, limit;
+  int64_t sorted_cap; // capacity of sorted_ids
   int m_major;       // workgroup order inside an XCD: all n-tiles of an m-block are neighbours
 };
 
@@ -451,27 +460,33 @@ __global__ __launch_bounds__(kThreads) void wstream_gemm_kernel(const GemmParams
 // Large-tile variant for compute-bound calls: 256 slots x 256 weight rows per
 // workgroup, one wavefront per SIMD, each owning a 128 x 128 register tile
 // (16 accumulator fragments in AGPRs), so one 16-byte fragment read from LDS
-// feeds four MFMAs.  K advances in 32-element tiles through a 4-stage LDS ring
-// filled by direct global->LDS loads (global_load_lds_dwordx4): three tiles are
-// in flight while one is consumed, and the only per-tile synchronisation is one
-// vmcnt wait plus one s_barrier.  The loads are issued from inline assembly so
-// that the vmcnt bookkeeping is exactly the one written here.
-// Staged rows are 64 bytes; 16-byte chunk c of row r sits at chunk
-// c ^ ((r >> 2) & 3), which makes both the DMA writes (4 lanes per row) and the
+// feeds four MFMAs.  The vector-memory path delivers 64 B/clk per CU against
+// 4096 MFMA flop/clk, so a tile needs >= 64 flop per loaded byte: 256 x 256
+// gives 128, and rows are staged 128 bytes (64 K elements) at a time because
+// a load that takes only half of a 128-byte line runs at half that rate.
+// K advances in 64-element tiles through two LDS stages filled by direct
+// global->LDS loads (global_load_lds_dwordx4, issued from inline assembly so
+// that no compiler-inserted wait serialises them): tile kt+2 is requested while
+// tile kt is being multiplied, and the only per-tile synchronisation is one
+// wait plus one s_barrier.  16-byte chunk c of row r sits at chunk
+// c ^ ((r >> 1) & 7), which makes both the DMA writes (8 lanes per row) and the
 // fragment reads (16 consecutive rows, one chunk) touch 16 distinct 16-byte
-// bank groups.  Token fragments holding only padding slots are skipped.
+// bank groups.  Token fragments holding only padding slots are skipped and
+// their rows are not loaded.
 // The epilogue rounds the accumulators to the activation dtype, parks the
 // wavefront's 128 x 128 tile in LDS and writes it out with 16-byte stores, the
 // gated activation being applied on the way.
 // ---------------------------------------------------------------------------
-constexpr int kBigBM = 256, kBigBNW = 256, kBigBK = 32, kBigStages = 4;
+constexpr int kBigBM = 256, kBigBNW = 256, kBigBK = 64, kBigStages = 2;
 constexpr int kBigRowBytes = kBigBK * 2;
 constexpr int kBigStageBytes = (kBigBM + kBigBNW) * kBigRowBytes;
-constexpr int kBigDmaPerTile = 8;            // global_load_lds instructions per thread and K tile
 constexpr int kEpiRowBytes = 128 * 2 + 16;   // one token row of a wavefront's tile, padded
 constexpr int kEpiWaveBytes = 128 * kEpiRowBytes;
 constexpr int kBigLdsBytes = 4 * kEpiWaveBytes > kBigStages * kBigStageBytes ? 4 * kEpiWaveBytes
                                                                               : kBigStages * kBigStageBytes;
+
+constexpr int kBigSideBytes = 2 * kBigBM * 4;  // per-slot token id and routed weight, kept for the epilogue
+constexpr int kBigLdsTotal = kBigLdsBytes + kBigSideBytes;
 
 typedef __attribute__((address_space(3))) char lds_char;
 
@@ -492,6 +507,14 @@ __device__ __forceinline__ void lds_dma16(const char* base, uint32_t lane_byte_o
       : "memory");
 }
 
+// Touches one dword of a line that a later tile will need, so that the line is
+// in L2 by the time the LDS DMA asks for it.  The value lands in `sink`, which
+// is threaded through every call and read once after the loop, so the register
+// stays reserved while such loads are in flight.
+__device__ __forceinline__ void l2_touch(const char* base, uint32_t lane_byte_offset, uint32_t& sink) {
+  asm volatile("global_load_dword %0, %1, %2" : "+v"(sink) : "v"(lane_byte_offset), "s"(base) : "memory");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
@@ -500,6 +523,14 @@ __device__ __forceinline__ void wait_vmcnt() {
 
 __device__ __forceinline__ void bare_barrier() {
   asm volatile("s_barrier" ::: "memory");
+}
+
+// x * sigmoid(x) with the hardware exp2 and reciprocal (about 1e-6 relative
+// error); the result is rounded to 16 bits right after, so it differs from the
+// exact-sequence moe_silu in well under one rounding in a thousand.
+__device__ __forceinline__ float silu_fast(float x) {
+  const float e = __builtin_amdgcn_exp2f(x * -1.44269504088896341f);
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
 template <typename El>
@@ -520,36 +551,42 @@ __device__ __forceinline__ uint32_t pack2<ElemF16>(float a, float b) {
 struct BigCtx {
   const char* a_base;   // wave-uniform base of the A rows
   const char* w_base;   // wave-uniform base of this expert's weights
-  uint32_t a_off[4];    // per-lane byte offsets of the four 64-row load groups
-  uint32_t w_off[4];
+  uint32_t a_off[8];    // per-lane byte offsets of the eight 32-row load groups
+  uint32_t w_off[8];
   uint32_t dma_lds;     // LDS offset of this wavefront's DMA window in stage 0, group 0
-  int rd_k[2];          // fragment read offsets for the two MFMA steps of a K tile
+  int a_groups;         // 32-row token groups that hold real slots
+  uint32_t pf_a_off;    // per-lane byte offset of token row `tid` (L2 prefetch)
+  uint32_t pf_w_off;    // per-lane byte offset of weight row `tid`
+  bool pf_a_live;       // token row `tid` holds a real slot
+  int rd_k[4];          // fragment read offsets for the four MFMA steps of a K tile
   int x_row;            // byte offset of this wavefront's first token row in a stage
   int w_row[4];         // byte offsets of this wavefront's weight fragments in a stage
 };
 
 // Main loop for a wavefront that has FMC live token fragments (0..4).
-// Schedule of one K tile (two MFMA steps, fragment sets P and Q in registers):
-//   read Q <- (kt, step 1) | 16 MFMAs on P | wait tile kt+1, barrier, issue tile
-//   kt+3 | read P <- (kt+1, step 0) | 16 MFMAs on Q
-// so the LDS reads of a step are always in flight behind the MFMAs of the
-// previous one.  sched_barrier keeps the compiler from re-serialising them.
+// One K tile is four MFMA steps; two register sets of fragments (P, Q)
+// alternate so that the LDS reads of a step are in flight behind the MFMAs of
+// the previous one:
+//   Q<-(kt,1) mma P | P<-(kt,2) mma Q | Q<-(kt,3) mma P |
+//   wait, barrier, request tile kt+2, P<-(kt+1,0) | mma Q
+// sched_barrier keeps the compiler from re-serialising reads and MFMAs.
 template <typename Mma, int FMC>
 __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, int nk,
                                              f32x16 (&acc)[4][4]) {
   auto issue_tile = [&](int kt) {
-    const uint32_t dst = c.dma_lds + (kt % kBigStages) * kBigStageBytes;
+    const uint32_t dst = c.dma_lds + (kt & 1) * kBigStageBytes;
     const char* ab = c.a_base + kt * kBigRowBytes;
     const char* wb = c.w_base + kt * kBigRowBytes;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) lds_dma16(ab, c.a_off[i], dst + i * 4096);
+    for (int i = 0; i < 8; ++i)
+      if (i < c.a_groups) lds_dma16(ab, c.a_off[i], dst + i * 4096);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) lds_dma16(wb, c.w_off[i], dst + (4 + i) * 4096);
+    for (int i = 0; i < 8; ++i) lds_dma16(wb, c.w_off[i], dst + (8 + i) * 4096);
   };
   constexpr int XF = FMC > 0 ? FMC : 1;
   auto read_frags = [&](int kt, int kk, uint4 (&wf)[4], uint4 (&xf)[XF]) {
     if constexpr (FMC > 0) {
-      const char* st = smem + (kt % kBigStages) * kBigStageBytes;
+      const char* st = smem + (kt & 1) * kBigStageBytes;
 #pragma unroll
       for (int fn = 0; fn < 4; ++fn) wf[fn] = *reinterpret_cast<const uint4*>(st + c.w_row[fn] + c.rd_k[kk]);
 #pragma unroll
@@ -564,14 +601,25 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
       for (int fn = 0; fn < 4; ++fn) acc[fn][fm] = Mma::mma(wf[fn], xf[fm], acc[fn][fm]);
   };
 
-  // tiles 0..2 in flight, tile 0 landed and visible, fragments of (0, step 0) requested
+  // Two L2 touches per thread and K tile, kPfAhead tiles ahead of the DMA (one
+  // token line, one weight line; 256 threads cover the 512 lines of a K tile).
+  // Exactly two are issued each time so that "all but the last two vector
+  // memory operations have returned" always means "the DMA of the next tile is
+  // complete".
+  constexpr int kPfAhead = 2;
+  uint32_t sink = 0;
+  auto touch_tile = [&](int kt) {
+    const int t = kt < nk ? kt : nk - 1;
+    l2_touch(c.a_base + t * kBigRowBytes, c.pf_a_off, sink);
+    l2_touch(c.w_base + t * kBigRowBytes, c.pf_w_off, sink);
+  };
+
   issue_tile(0);
-  if (1 < nk) issue_tile(1);
-  if (2 < nk) issue_tile(2);
-  if (2 < nk) wait_vmcnt<2 * kBigDmaPerTile>();
-  else if (1 < nk) wait_vmcnt<kBigDmaPerTile>();
-  else wait_vmcnt<0>();
+  wait_vmcnt<0>();
   bare_barrier();
+  if (1 < nk) issue_tile(1);
+  touch_tile(2);
+  touch_tile(3);
   uint4 wfP[4], xfP[XF], wfQ[4], xfQ[XF];
   read_frags(0, 0, wfP, xfP);
   __builtin_amdgcn_sched_barrier(0);
@@ -581,18 +629,30 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
     __builtin_amdgcn_sched_barrier(0);
     mma_all(wfP, xfP);
     __builtin_amdgcn_sched_barrier(0);
+    read_frags(kt, 2, wfP, xfP);
+    __builtin_amdgcn_sched_barrier(0);
+    mma_all(wfQ, xfQ);
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(kt, 3, wfQ, xfQ);
+    __builtin_amdgcn_sched_barrier(0);
+    mma_all(wfP, xfP);
+    __builtin_amdgcn_sched_barrier(0);
     if (kt + 1 < nk) {
-      // tile kt+1 must have landed; tile kt+2 may still be in flight
-      if (kt + 2 < nk) wait_vmcnt<kBigDmaPerTile>();
-      else wait_vmcnt<0>();
+      // tile kt+1 has landed (everything but the two newest touches has
+      // returned) and nobody reads stage kt any more (the reads of step 3 have
+      // returned: lgkmcnt(0)) -> it can take tile kt+2
+      asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
       bare_barrier();
-      if (kt + 3 < nk) issue_tile(kt + 3);  // into the stage of tile kt-1, fully consumed
+      if (kt + 2 < nk) issue_tile(kt + 2);
+      touch_tile(kt + 2 + kPfAhead);
       read_frags(kt + 1, 0, wfP, xfP);
     }
     __builtin_amdgcn_sched_barrier(0);
     mma_all(wfQ, xfQ);
     __builtin_amdgcn_sched_barrier(0);
   }
+  wait_vmcnt<0>();
+  asm volatile("" ::"v"(sink));
 }
 
 // Epilogue phase 1: round this wavefront's accumulators to the activation dtype
@@ -600,16 +660,12 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
 // as [token row][weight row].
 template <typename El, int FMC, bool GATED>
 __device__ __forceinline__ void big_park(const GemmParams& p, int e, int n0, int wn, int lhi, int l32,
-                                         int slot0, char* epi, const f32x16 (&acc)[4][4]) {
+                                         const float* s_rw, char* epi, const f32x16 (&acc)[4][4]) {
   using S = typename El::S;
   const S* bias = static_cast<const S*>(p.bias);
 #pragma unroll
   for (int fm = 0; fm < FMC; ++fm) {
-    float rw = 1.f;
-    if (p.mul_weight) {
-      const int tok = p.sorted_ids[slot0 + fm * 32 + l32];
-      rw = tok < p.numel ? p.topk_w[tok] : 0.f;
-    }
+    const float rw = s_rw[fm * 32 + l32];  // 1 when the routed weight is not applied here
     char* row = epi + (fm * 32 + l32) * kEpiRowBytes;
 #pragma unroll
     for (int fn = 0; fn < 4; ++fn) {
@@ -651,7 +707,7 @@ __device__ __forceinline__ void big_park(const GemmParams& p, int e, int n0, int
 // the matching up values.
 template <typename El, bool GATED>
 __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, int lane, int slot0,
-                                          int rows, const char* epi) {
+                                          int rows, const int* s_tok, const char* epi) {
   using S = typename El::S;
   constexpr int COLS = GATED ? 64 : 128;      // output columns of the wavefront tile
   constexpr int LPR = COLS / 8;               // lanes per row
@@ -662,7 +718,7 @@ __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, i
     const int r = r0 + lane / LPR;
     if (r >= rows) continue;
     const int slot = slot0 + r;
-    const int tok = p.sorted_ids[slot];
+    const int tok = s_tok[r];
     if (tok >= p.numel) continue;
     const char* row = epi + r * kEpiRowBytes;
     uint4 out;
@@ -680,7 +736,7 @@ __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, i
           const float uv = El::ld(static_cast<S>(uw[i] >> (16 * hlf)));
           float rr;
           if (p.activation == MOE_ACT_SILU) {
-            rr = El::ld(El::st(moe_silu(gv))) * uv;
+            rr = El::ld(El::st(silu_fast(gv))) * uv;
           } else if (p.activation == MOE_ACT_SWIGLUOAI) {
             rr = moe_swigluoai(gv, uv, p.alpha, p.limit);
           } else {
@@ -710,7 +766,8 @@ __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, i
 
 template <typename Mma, int FMC, bool GATED>
 __device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, char* smem, int nk,
-                                         int e, int n0, int wn, int lane, int slot0, char* epi) {
+                                         int e, int n0, int wn, int lane, float my_rw, float* s_rw_all,
+                                         const float* s_rw, char* epi) {
   using El = typename Mma::El;
   f32x16 acc[4][4];
 #pragma unroll
@@ -720,8 +777,10 @@ __device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, c
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[fn][fm][r] = 0.f;
   big_mainloop<Mma, FMC>(c, smem, nk, acc);
+  s_rw_all[threadIdx.x] = my_rw;  // requested before the main loop, needed only now
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   bare_barrier();  // every wavefront is done reading the stages before they are reused
-  if constexpr (FMC > 0) big_park<El, FMC, GATED>(p, e, n0, wn, lane >> 5, lane & 31, slot0, epi, acc);
+  if constexpr (FMC > 0) big_park<El, FMC, GATED>(p, e, n0, wn, lane >> 5, lane & 31, s_rw, epi, acc);
 }
 
 template <typename Mma, bool GATED>
@@ -739,32 +798,61 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
     nt = logical / p.num_m_blocks;
     mb = logical - nt * p.num_m_blocks;
   }
-  if (mb * kBigBM >= *p.num_post_pad) return;
-  const int e = p.expert_ids[mb];
-  const int n0 = nt * (GATED ? kBigBNW / 2 : kBigBNW);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lhi = lane >> 5;
   const int wm = wave & 1, wn = wave >> 1;
+  [[maybe_unused]] const unsigned long long t_start = MOE_TRACE_NOW();
+  // the three loads below do not depend on each other: one memory latency, not three
+  const int npp = *p.num_post_pad;
+  const int e = p.expert_ids[mb];
+  const int64_t my_slot = static_cast<int64_t>(mb) * kBigBM + tid;
+  const int my_tok = p.sorted_ids[my_slot < p.sorted_cap ? my_slot : p.sorted_cap - 1];
+  if (mb * kBigBM >= npp) return;
+  const int n0 = nt * (GATED ? kBigBNW / 2 : kBigBNW);
+  int* s_tok = reinterpret_cast<int*>(smem + kBigLdsBytes);
+  float* s_rw_all = reinterpret_cast<float*>(smem + kBigLdsBytes + kBigBM * 4);
+  s_tok[tid] = my_tok;
   // real slots come first in a block
-  const int my_tok = p.sorted_ids[mb * kBigBM + tid];
   const int nvalid = __syncthreads_count(my_tok < p.numel);
   if (nvalid == 0) return;
+  float my_rw = 1.f;
+  if (p.mul_weight) my_rw = my_tok < p.numel ? p.topk_w[my_tok] : 0.f;
 
   BigCtx c;
-  const int ld_row = tid >> 2;                        // row inside a 64-row load group
-  const int ld_chunk = (tid & 3) ^ ((tid >> 4) & 3);  // logical chunk this lane fetches
+  const int ld_row = tid >> 3;                        // row inside a 32-row load group
+  const int ld_chunk = (tid & 7) ^ ((tid >> 4) & 7);  // logical chunk this lane fetches
   c.a_base = static_cast<const char*>(p.a);
   c.w_base = static_cast<const char*>(p.w) + static_cast<int64_t>(e) * p.w_stride_e * 2;
+  c.a_groups = (nvalid + 31) >> 5;
+  {
+    // L2 prefetch: this thread owns token row `tid` and weight row `tid` of the tile
+    const int tok = my_tok;
+    const int64_t src = p.a_by_slot ? static_cast<int64_t>(mb * kBigBM + tid)
+                                    : (tok < p.numel ? tok / p.top_k : 0);
+    c.pf_a_off = static_cast<uint32_t>(src * p.lda * 2);
+    c.pf_a_live = tok < p.numel;
+    int64_t wrow;
+    if constexpr (GATED) {
+      const int half = tid >> 7;
+      int n = n0 + (tid & 127);
+      n = n < p.N ? n : p.N - 1;
+      wrow = p.interleaved ? (2 * n + half) : (half * p.N + n);
+    } else {
+      const int n = n0 + tid;
+      wrow = n < p.N ? n : p.N - 1;
+    }
+    c.pf_w_off = static_cast<uint32_t>(wrow * p.w_stride_n * 2);
+  }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int slot = mb * kBigBM + ld_row + 64 * i;
+  for (int i = 0; i < 8; ++i) {
+    const int slot = mb * kBigBM + ld_row + 32 * i;
     int64_t src = slot;
     if (!p.a_by_slot) {
-      const int tok = p.sorted_ids[slot];
+      const int tok = s_tok[ld_row + 32 * i];
       src = tok < p.numel ? tok / p.top_k : 0;
     }
     c.a_off[i] = static_cast<uint32_t>((src * p.lda + ld_chunk * 8) * 2);
-    const int rr = ld_row + 64 * i;
+    const int rr = ld_row + 32 * i;
     int64_t wrow;
     if constexpr (GATED) {
       const int half = rr >> 7;
@@ -779,7 +867,7 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   }
   c.dma_lds = __builtin_amdgcn_readfirstlane(lds_offset_of(smem) + wave * 1024);
 #pragma unroll
-  for (int kk = 0; kk < 2; ++kk) c.rd_k[kk] = l32 * kBigRowBytes + (((2 * kk + lhi) ^ ((l32 >> 2) & 3)) << 4);
+  for (int kk = 0; kk < 4; ++kk) c.rd_k[kk] = l32 * kBigRowBytes + (((2 * kk + lhi) ^ ((l32 >> 1) & 7)) << 4);
   c.x_row = wm * 128 * kBigRowBytes;
 #pragma unroll
   for (int fn = 0; fn < 4; ++fn) {
@@ -793,20 +881,30 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   const int nk = p.Kd / kBigBK;
   const int slot0 = mb * kBigBM + wm * 128;
   char* epi = smem + wave * kEpiWaveBytes;
+  [[maybe_unused]] const unsigned long long t_pro = MOE_TRACE_NOW();
   const int rows = min(128, max(0, nvalid - wm * 128));  // real slots of this wavefront
   switch ((rows + 31) >> 5) {
-    case 0: big_wave<Mma, 0, GATED>(p, c, smem, nk, e, n0, wn, lane, slot0, epi); break;
-    case 1: big_wave<Mma, 1, GATED>(p, c, smem, nk, e, n0, wn, lane, slot0, epi); break;
-    case 2: big_wave<Mma, 2, GATED>(p, c, smem, nk, e, n0, wn, lane, slot0, epi); break;
-    case 3: big_wave<Mma, 3, GATED>(p, c, smem, nk, e, n0, wn, lane, slot0, epi); break;
-    default: big_wave<Mma, 4, GATED>(p, c, smem, nk, e, n0, wn, lane, slot0, epi); break;
+    case 0: big_wave<Mma, 0, GATED>(p, c, smem, nk, e, n0, wn, lane, my_rw, s_rw_all, s_rw_all + wm * 128, epi); break;
+    case 1: big_wave<Mma, 1, GATED>(p, c, smem, nk, e, n0, wn, lane, my_rw, s_rw_all, s_rw_all + wm * 128, epi); break;
+    case 2: big_wave<Mma, 2, GATED>(p, c, smem, nk, e, n0, wn, lane, my_rw, s_rw_all, s_rw_all + wm * 128, epi); break;
+    case 3: big_wave<Mma, 3, GATED>(p, c, smem, nk, e, n0, wn, lane, my_rw, s_rw_all, s_rw_all + wm * 128, epi); break;
+    default: big_wave<Mma, 4, GATED>(p, c, smem, nk, e, n0, wn, lane, my_rw, s_rw_all, s_rw_all + wm * 128, epi); break;
   }
-  big_flush<El, GATED>(p, n0, wn, lane, slot0, rows, epi);
+  [[maybe_unused]] const unsigned long long t_main = MOE_TRACE_NOW();
+  big_flush<El, GATED>(p, n0, wn, lane, slot0, rows, s_tok + wm * 128, epi);
+#ifdef MOE_TRACE
+  const unsigned long long t_end = MOE_TRACE_NOW();
+  if (tid == 0 && blockIdx.x < 4096) {
+    moe_dbg[blockIdx.x * 8 + 0] = t_start; moe_dbg[blockIdx.x * 8 + 1] = t_pro;
+    moe_dbg[blockIdx.x * 8 + 2] = t_main; moe_dbg[blockIdx.x * 8 + 3] = t_end;
+    moe_dbg[blockIdx.x * 8 + 4] = nvalid; moe_dbg[blockIdx.x * 8 + 5] = __builtin_amdgcn_s_getreg((20) | (0 << 6) | (3 << 11));
+  }
+#endif
 }
 
 template <typename Mma, bool GATED>
 int launch_big(GemmParams& p, int64_t sorted_cap, hipStream_t s) {
-  constexpr int lds = kBigLdsBytes;
+  constexpr int lds = kBigLdsTotal;
   auto kern = big_gemm_kernel<Mma, GATED>;
   static bool attr_set = false;
   if (!attr_set) {
@@ -969,12 +1067,13 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.num_post_pad = a->num_tokens_post_pad;
   p.topk_w = a->topk_weights;
   p.numel = static_cast<int>(numel);
+  p.sorted_cap = a->sorted_cap;
   p.top_k = a->K;
   p.alpha = a->swiglu_alpha;
   p.limit = a->swiglu_limit;
   p.activation = a->activation;
   p.interleaved = a->activation == MOE_ACT_SWIGLUOAI;
-  p.m_major = getenv("MOE_MAP") ? atoi(getenv("MOE_MAP")) : 0;
+  p.m_major = getenv("MOE_MAP") ? atoi(getenv("MOE_MAP")) : 1;
 
   // pass 1: x . W13^T with the gated activation, rows addressed by slot
   p.a = a->x; p.lda = a->H; p.w = a->w13; p.w_stride_e = a->w13_stride_e; p.w_stride_n = a->w13_stride_n;
@@ -1002,3 +1101,9 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   if (!(passes & 4)) return MOE_OK;
   return moe_sum(a->out, c3, a->T, a->K, a->H, a->act_dtype, a->stream);
 }
+
+#ifdef MOE_TRACE
+MOE_EXPORT int moe_debug_read(void* dst, int64_t bytes) {
+  return hipMemcpyFromSymbol(dst, HIP_SYMBOL(moe_dbg), bytes) == hipSuccess ? 0 : -1;
+}
+#endif
