@@ -71,6 +71,7 @@ struct GemmParams {
   int interleaved;   // gate/up rows interleaved (2n, 2n+1) instead of halves (n, N+n)
   float alpha, limit;
   int64_t sorted_cap; // capacity of sorted_ids
+  int align_bs;      // block size the alignment was made with (a multiple of the kernel's M tile)
   int m_major;       // workgroup order inside an XCD: all n-tiles of an m-block are neighbours
 };
 
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     mb = logical - nt * p.num_m_blocks;
   }
   if (mb * BM >= *p.num_post_pad) return;
-  const int e = p.expert_ids[mb];
+  const int e = p.expert_ids[(mb * BM) / p.align_bs];
   const int n0 = nt * BN_OUT;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -292,169 +293,6 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
   }
 }
 
-
-// ---------------------------------------------------------------------------
-// Weight-streaming variant.  The token tile (BM = 32*FM rows) is shared by the
-// four wavefronts through LDS; every wavefront owns 64 weight rows of the strip
-// (32 gate + 32 up rows of the same output columns when gated) and loads them
-// from global memory straight into registers, 64 contiguous bytes per lane and
-// K tile, WDEPTH K tiles ahead.  Weights therefore never pass through LDS, and
-// one token fragment read from LDS feeds two MFMAs.  Lane (r, h) of a weight
-// fragment holds K elements [32h, 32h+32) of the 64-wide K tile, so MFMA step j
-// multiplies 16-byte chunk 4h+j of both operands (any pairing of K elements is
-// a valid dot product as long as both operands use the same one).
-// Token fragments that hold only padding slots are skipped.
-// ---------------------------------------------------------------------------
-template <typename Mma, int FM, int WDEPTH, bool GATED>
-__global__ __launch_bounds__(kThreads) void wstream_gemm_kernel(const GemmParams p) {
-  using El = typename Mma::El;
-  constexpr int BM = FM * 32;
-  constexpr int NOUT_WAVE = GATED ? 32 : 64;  // output columns per wavefront
-  constexpr int BN_OUT = 4 * NOUT_WAVE;
-  constexpr int STAGE_BYTES = BM * kRowBytes;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-
-  const int per_xcd = gridDim.x / kXcds;
-  const int logical = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
-  if (logical >= p.num_m_blocks * p.num_n_tiles) return;
-  int nt, mb;
-  if (p.m_major) {
-    mb = logical / p.num_n_tiles;
-    nt = logical - mb * p.num_n_tiles;
-  } else {
-    nt = logical / p.num_m_blocks;
-    mb = logical - nt * p.num_m_blocks;
-  }
-  if (mb * BM >= *p.num_post_pad) return;
-  const int e = p.expert_ids[mb];
-  const int n0 = nt * BN_OUT;
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int l32 = lane & 31, lhi = lane >> 5;
-  const int ld_row = tid >> 3, ld_c = tid & 7;
-
-  // real slots come first in a block: count them, whole fragments past them are skipped
-  int my_tok = p.numel;
-  if (tid < BM) my_tok = p.sorted_ids[mb * BM + tid];
-  const int nvalid = __syncthreads_count(my_tok < p.numel);
-  const int fm_eff = (nvalid + 31) >> 5;
-  if (fm_eff == 0) return;
-
-  const char* a_src[FM];
-#pragma unroll
-  for (int j = 0; j < FM; ++j) {
-    const int slot = mb * BM + ld_row + 32 * j;
-    int64_t src = slot;
-    if (!p.a_by_slot) {
-      const int tok = p.sorted_ids[slot];
-      src = tok < p.numel ? tok / p.top_k : 0;
-    }
-    a_src[j] = static_cast<const char*>(p.a) + (src * p.lda + ld_c * 8) * 2;
-  }
-  const char* w_src[2];
-#pragma unroll
-  for (int f = 0; f < 2; ++f) {
-    int64_t wrow;
-    if constexpr (GATED) {
-      int n = n0 + wave * 32 + l32;
-      n = n < p.N ? n : p.N - 1;
-      wrow = p.interleaved ? (2 * n + f) : (f * p.N + n);
-    } else {
-      const int n = n0 + wave * 64 + f * 32 + l32;
-      wrow = n < p.N ? n : p.N - 1;
-    }
-    w_src[f] = static_cast<const char*>(p.w) +
-               (static_cast<int64_t>(e) * p.w_stride_e + wrow * p.w_stride_n + lhi * 32) * 2;
-  }
-  const int st_off = swizzled(ld_row, ld_c);
-  int rd_k[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) rd_k[j] = l32 * kRowBytes + (((4 * lhi + j) ^ ((l32 >> 1) & 7)) << 4);
-
-  f32x16 acc[2][FM];
-#pragma unroll
-  for (int f = 0; f < 2; ++f)
-#pragma unroll
-    for (int fm = 0; fm < FM; ++fm)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[f][fm][r] = 0.f;
-
-  uint4 t_reg[FM];
-  uint4 w_reg[WDEPTH][2][4];
-  const int nk = (p.Kd + kBK - 1) / kBK;
-  const bool k_exact = (p.Kd % kBK) == 0;
-
-  auto load_tokens = [&](int kt) {
-    const bool in_k = k_exact || kt * kBK + ld_c * 8 < p.Kd;
-#pragma unroll
-    for (int j = 0; j < FM; ++j)
-      if (j < fm_eff)
-        t_reg[j] = in_k ? *reinterpret_cast<const uint4*>(a_src[j] + kt * kRowBytes) : uint4{0, 0, 0, 0};
-  };
-  auto store_tokens = [&](int stage) {
-    char* base = smem + stage * STAGE_BYTES + st_off;
-#pragma unroll
-    for (int j = 0; j < FM; ++j)
-      if (j < fm_eff) *reinterpret_cast<uint4*>(base + j * 32 * kRowBytes) = t_reg[j];
-  };
-  auto load_weights = [&](int kt, uint4 (&dst)[2][4]) {
-#pragma unroll
-    for (int f = 0; f < 2; ++f)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const bool in_k = k_exact || kt * kBK + lhi * 32 + j * 8 < p.Kd;
-        dst[f][j] = in_k ? *reinterpret_cast<const uint4*>(w_src[f] + kt * kRowBytes + j * 16)
-                         : uint4{0, 0, 0, 0};
-      }
-  };
-
-  // prologue: weights for tiles 0 .. WDEPTH-2, tokens for tile 0
-#pragma unroll
-  for (int d = 0; d < WDEPTH - 1; ++d)
-    if (d < nk) load_weights(d, w_reg[d]);
-  load_tokens(0);
-  store_tokens(0);
-  __syncthreads();
-
-  for (int kt0 = 0; kt0 < nk; kt0 += WDEPTH) {
-#pragma unroll
-    for (int d = 0; d < WDEPTH; ++d) {
-      const int kt = kt0 + d;
-      if (kt < nk) {
-        if (kt + WDEPTH - 1 < nk) load_weights(kt + WDEPTH - 1, w_reg[(d + WDEPTH - 1) % WDEPTH]);
-        if (kt + 1 < nk) load_tokens(kt + 1);
-        const char* st = smem + (kt & 1) * STAGE_BYTES;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-#pragma unroll
-          for (int fm = 0; fm < FM; ++fm) {
-            if (fm < fm_eff) {
-              const uint4 xf = *reinterpret_cast<const uint4*>(st + fm * 32 * kRowBytes + rd_k[j]);
-              acc[0][fm] = Mma::mma(w_reg[d][0][j], xf, acc[0][fm]);
-              acc[1][fm] = Mma::mma(w_reg[d][1][j], xf, acc[1][fm]);
-            }
-          }
-        }
-        if (kt + 1 < nk) store_tokens((kt + 1) & 1);
-        __syncthreads();
-      }
-    }
-  }
-
-#pragma unroll
-  for (int fm = 0; fm < FM; ++fm) {
-    if (fm >= fm_eff) continue;
-    const int slot = mb * BM + fm * 32 + l32;
-    const int tok = p.sorted_ids[slot];
-    if (tok >= p.numel) continue;
-    if constexpr (GATED) {
-      store_fragment<El, true>(p, e, acc[0][fm], acc[1][fm], tok, slot, n0 + wave * 32 + 4 * lhi);
-    } else {
-      store_fragment<El, false>(p, e, acc[0][fm], acc[0][fm], tok, slot, n0 + wave * 64 + 4 * lhi);
-      store_fragment<El, false>(p, e, acc[1][fm], acc[1][fm], tok, slot, n0 + wave * 64 + 32 + 4 * lhi);
-    }
-  }
-}
 
 // ---------------------------------------------------------------------------
 // Large-tile variant for compute-bound calls: 256 slots x 256 weight rows per
@@ -804,7 +642,7 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   [[maybe_unused]] const unsigned long long t_start = MOE_TRACE_NOW();
   // the three loads below do not depend on each other: one memory latency, not three
   const int npp = *p.num_post_pad;
-  const int e = p.expert_ids[mb];
+  const int e = p.expert_ids[(mb * kBigBM) / p.align_bs];
   const int64_t my_slot = static_cast<int64_t>(mb) * kBigBM + tid;
   const int my_tok = p.sorted_ids[my_slot < p.sorted_cap ? my_slot : p.sorted_cap - 1];
   if (mb * kBigBM >= npp) return;
@@ -923,30 +761,6 @@ int launch_big(GemmParams& p, int64_t sorted_cap, hipStream_t s) {
   return moe_check_launch(GATED ? "fused_experts (gate-up pass)" : "fused_experts (down pass)");
 }
 
-template <typename Mma, int FM, int WDEPTH, bool GATED>
-int launch_wstream(GemmParams& p, int64_t sorted_cap, hipStream_t s) {
-  constexpr int BM = FM * 32;
-  constexpr int lds = 2 * BM * kRowBytes;
-  constexpr int bn_out = GATED ? 128 : 256;
-  p.num_m_blocks = static_cast<int>((sorted_cap + BM - 1) / BM);
-  p.num_n_tiles = (p.N + bn_out - 1) / bn_out;
-  auto kern = wstream_gemm_kernel<Mma, FM, WDEPTH, GATED>;
-  const int64_t tiles = static_cast<int64_t>(p.num_m_blocks) * p.num_n_tiles;
-  const int64_t grid = (tiles + kXcds - 1) / kXcds * kXcds;
-  if (grid > INT32_MAX) return moe_fail(MOE_ERR_ARG, "fused_experts: grid of %lld workgroups", static_cast<long long>(grid));
-  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(kThreads), lds, s, p);
-  return moe_check_launch(GATED ? "fused_experts (gate-up pass)" : "fused_experts (down pass)");
-}
-
-int gemm_variant() {
-  static int v = -1;
-  if (v < 0) {
-    const char* e = getenv("MOE_GEMM_VARIANT");
-    v = e ? atoi(e) : 0;
-  }
-  return v;
-}
-
 template <typename Mma, int BM, int BNW, int WAVES_M, bool GATED>
 int launch(const GemmParams& p, hipStream_t s) {
   constexpr int lds = 2 * (BM + BNW) * kRowBytes;
@@ -966,33 +780,29 @@ int launch(const GemmParams& p, hipStream_t s) {
   return moe_check_launch(GATED ? "fused_experts (gate-up pass)" : "fused_experts (down pass)");
 }
 
+// Picks the largest M tile that divides the caller's alignment block size: a
+// block of the aligned list is then a whole number of kernel tiles, all of one
+// expert.
 template <typename Mma, bool GATED>
 int launch_bm(GemmParams& p, int block_size, int64_t sorted_cap, hipStream_t s) {
-  if (block_size == 256 && p.Kd % kBigBK == 0 && gemm_variant() != 2) return launch_big<Mma, GATED>(p, sorted_cap, s);
-  if (gemm_variant() == 2) {
-    switch (block_size) {
-      case 256: return launch_wstream<Mma, 8, 2, GATED>(p, sorted_cap, s);
-      case 128: return launch_wstream<Mma, 4, 2, GATED>(p, sorted_cap, s);
-      case 64: return launch_wstream<Mma, 2, 3, GATED>(p, sorted_cap, s);
-      case 32: return launch_wstream<Mma, 1, 4, GATED>(p, sorted_cap, s);
-      default:
-        return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: block_size %d (supported: 32, 64, 128, 256)", block_size);
-    }
+  p.align_bs = block_size;
+  if (block_size % 256 == 0 && p.Kd % kBigBK == 0) return launch_big<Mma, GATED>(p, sorted_cap, s);
+  if (block_size % 128 == 0) {
+    p.num_m_blocks = static_cast<int>((sorted_cap + 127) / 128);
+    p.num_n_tiles = (p.N + (GATED ? 64 : 128) - 1) / (GATED ? 64 : 128);
+    return launch<Mma, 128, 128, 2, GATED>(p, s);
   }
-  p.num_m_blocks = static_cast<int>((sorted_cap + block_size - 1) / block_size);
-  switch (block_size) {
-    case 128:
-      p.num_n_tiles = (p.N + (GATED ? 64 : 128) - 1) / (GATED ? 64 : 128);
-      return launch<Mma, 128, 128, 2, GATED>(p, s);
-    case 64:
-      p.num_n_tiles = (p.N + (GATED ? 128 : 256) - 1) / (GATED ? 128 : 256);
-      return launch<Mma, 64, 256, 1, GATED>(p, s);
-    case 32:
-      p.num_n_tiles = (p.N + (GATED ? 128 : 256) - 1) / (GATED ? 128 : 256);
-      return launch<Mma, 32, 256, 1, GATED>(p, s);
-    default:
-      return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: block_size %d (supported: 32, 64, 128)", block_size);
+  if (block_size % 64 == 0) {
+    p.num_m_blocks = static_cast<int>((sorted_cap + 63) / 64);
+    p.num_n_tiles = (p.N + (GATED ? 128 : 256) - 1) / (GATED ? 128 : 256);
+    return launch<Mma, 64, 256, 1, GATED>(p, s);
   }
+  if (block_size % 32 == 0) {
+    p.num_m_blocks = static_cast<int>((sorted_cap + 31) / 32);
+    p.num_n_tiles = (p.N + (GATED ? 128 : 256) - 1) / (GATED ? 128 : 256);
+    return launch<Mma, 32, 256, 1, GATED>(p, s);
+  }
+  return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: block_size %d is not a multiple of 32", block_size);
 }
 
 int elem_size(int dtype) { return dtype == MOE_F32 ? 4 : (dtype == MOE_E4M3 ? 1 : 2); }
@@ -1004,6 +814,7 @@ MOE_EXPORT int moe_preferred_block_size(int M, int E, int K, int act_dtype, int 
   (void)weight_dtype;
   if (E < 1) return 64;
   const int64_t avg = static_cast<int64_t>(M) * K / E;  // routed rows per expert
+  if (avg >= 256) return 256;
   if (avg >= 96) return 128;
   if (avg >= 24) return 64;
   return 32;
@@ -1073,7 +884,9 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.limit = a->swiglu_limit;
   p.activation = a->activation;
   p.interleaved = a->activation == MOE_ACT_SWIGLUOAI;
-  p.m_major = getenv("MOE_MAP") ? atoi(getenv("MOE_MAP")) : 1;
+  // the large-tile kernel reuses a token block across its n-tiles in one L2;
+  // the small-block kernels stream weights and keep a weight strip in one L2
+  p.m_major = (a->block_size % 256 == 0 && a->H % kBigBK == 0 && a->I % kBigBK == 0) ? 1 : 0;
 
   // pass 1: x . W13^T with the gated activation, rows addressed by slot
   p.a = a->x; p.lda = a->H; p.w = a->w13; p.w_stride_e = a->w13_stride_e; p.w_stride_n = a->w13_stride_n;

@@ -42,7 +42,7 @@ def test_fused_experts_against_oracle(moe, oracle, dev, dtype, E, H, I, T, K):
     _close(out, mirrored, rtol=1.6e-2, atol=2e-3)
 
 
-@pytest.mark.parametrize("bm", [32, 64, 128, 256])
+@pytest.mark.parametrize("bm", [32, 64, 96, 128, 256, 512])
 def test_every_block_size_kernel(moe, oracle, dev, bm, monkeypatch):
     x, w13, w2, logits = _layer(16, 256, 128, 500, 4, 5, torch.bfloat16)
     tw, ids, _ = oracle.topk_softmax(logits, 4, renormalize=True)
