@@ -32,8 +32,9 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs (summaries under profiles/); None until measured.
-MEASURED_TRAFFIC_BYTES = {"layered_8192p_256d": None, "decode_256": None}
+# WRITE_SIZE runs (profiles/hbm_traffic_gate_up_kernels.txt): fetch + write bytes.
+MEASURED_TRAFFIC_BYTES = {"layered_8192p_256d": 1693171712 + 144224256,
+                          "decode_256": 518821888 + 3155968}
 
 
 def _events(n):
@@ -111,6 +112,55 @@ def time_stages(layer: Layer, steps: int):
     return {n: statistics.fmean(v) for n, v in per.items()}, ids
 
 
+def chunk_amplification(moe, layer: "Layer", reps: int, mode: str = "both"):
+    """Config 4: the 8192-token prompt as 16 chunks of 512 tokens, each co-batched
+    with the 256 decode tokens (16 calls of T=768), against the single 8192+256
+    pass on the same layer.  Chunked prefill streams every active expert's
+    weights once per chunk; the layered pass streams them once."""
+    wl, s = moe.workloads, layer.shape
+    dec = torch.arange(8192, 8448, device=layer.dev)
+    chunks = []
+    for c in range(16):
+        sel = torch.cat([torch.arange(c * 512, (c + 1) * 512, device=layer.dev), dec])
+        chunks.append((layer.x[sel].contiguous(), layer.logits[sel].contiguous()))
+
+    def run_chunked():
+        act = 0
+        for xc, lc in chunks:
+            tw, ids, _ = moe.fused_topk(xc, lc, s.top_k, True)
+            moe.fused_experts(xc, layer.w13, layer.w2, None, None, tw, ids)
+        return act
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        ev = _events(2)
+        ev[0].record()
+        for _ in range(reps):
+            fn()
+        ev[1].record()
+        torch.cuda.synchronize()
+        return ev[0].elapsed_time(ev[1]) / reps
+
+    out = {}
+    per_expert = 3 * s.hidden * s.intermediate * 2
+    if mode in ("both", "chunked"):
+        out["chunked_16x(512+256)_ms"] = round(timed(run_chunked), 4)
+        act = 0
+        for xc, lc in chunks:
+            _, ids, _ = moe.fused_topk(xc, lc, s.top_k, True)
+            act += int(torch.unique(ids).numel())
+        out["chunked_expert_weight_bytes"] = act * per_expert
+    if mode in ("both", "single"):
+        out["single_pass_ms"] = round(timed(layer.step), 4)
+        _, ids, _ = moe.fused_topk(layer.x, layer.logits, s.top_k, True)
+        out["single_expert_weight_bytes"] = int(torch.unique(ids).numel()) * per_expert
+    if mode == "both":
+        out["time_ratio"] = round(out["chunked_16x(512+256)_ms"] / out["single_pass_ms"], 3)
+        out["weight_bytes_ratio"] = round(out["chunked_expert_weight_bytes"] / out["single_expert_weight_bytes"], 3)
+    return out
+
+
 def cpu_baseline(moe, name: str, runs: int):
     """The oracle (PyTorch fp32 restatement of the reference's MoE math; bf16
     weights upcast per expert) on this host's cores: bounded sample."""
@@ -145,6 +195,14 @@ def main() -> int:
                     choices=["layered_8192p_256d", "decode_256"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-runs", type=int, default=2)
+    ap.add_argument("--chunk-mode", default="both", choices=["both", "chunked", "single", "off"],
+                    help="config 4 (chunk amplification) leg: both sides, one side only (for "
+                         "rocprofv3 counter runs), or off")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three plain 1 GiB device copies, the known-size kernel that "
+                         "FETCH_SIZE / WRITE_SIZE readings are scaled by")
+    ap.add_argument("--only-chunk-leg", action="store_true",
+                    help="run nothing but the chunk-amplification leg")
     ap.add_argument("--block-size-m", type=int, default=0,
                     help="override the alignment block size (0 = the library's choice)")
     a = ap.parse_args()
@@ -163,7 +221,18 @@ def main() -> int:
     if a.block_size_m:
         moe.fused_moe.try_get_optimal_moe_config = lambda *x, **k: {"BLOCK_SIZE_M": a.block_size_m}
         moe.try_get_optimal_moe_config = moe.fused_moe.try_get_optimal_moe_config
+    if a.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     main_layer = Layer(moe, a.workload, dev)
+    if a.only_chunk_leg:
+        print(json.dumps({"chunk_amplification": chunk_amplification(moe, main_layer, max(2, a.steps // 10),
+                                                                      a.chunk_mode)}))
+        return 0
     ms = time_steps(main_layer, a.steps, a.warmup)
     stages, ids = time_stages(main_layer, max(5, a.steps // 2))
     shape = main_layer.shape
@@ -208,6 +277,8 @@ def main() -> int:
         "roofline": roofline,
     }
 
+    if compute_bound and a.chunk_mode != "off":
+        out["chunk_amplification"] = chunk_amplification(moe, main_layer, max(2, a.steps // 10), a.chunk_mode)
     if compute_bound:
         dec = Layer(moe, "decode_256", dev)
         dms = time_steps(dec, max(a.steps, 50), max(a.warmup, 10))

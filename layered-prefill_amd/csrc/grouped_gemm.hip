@@ -21,7 +21,7 @@
 
 #ifdef MOE_TRACE
 // Development aid (make EXTRA=-DMOE_TRACE): per-workgroup phase timestamps of the large-tile kernel.
-__device__ unsigned long long moe_dbg[8 * 4096];
+__device__ unsigned long long moe_dbg[8 * 4096 + 4 * 128];
 #define MOE_TRACE_NOW() __builtin_amdgcn_s_memrealtime()
 #else
 #define MOE_TRACE_NOW() 0ull
@@ -302,29 +302,33 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
 // 4096 MFMA flop/clk, so a tile needs >= 64 flop per loaded byte: 256 x 256
 // gives 128, and rows are staged 128 bytes (64 K elements) at a time because
 // a load that takes only half of a 128-byte line runs at half that rate.
-// K advances in 64-element tiles through two LDS stages filled by direct
-// global->LDS loads (global_load_lds_dwordx4, issued from inline assembly so
-// that no compiler-inserted wait serialises them): tile kt+2 is requested while
-// tile kt is being multiplied, and the only per-tile synchronisation is one
-// wait plus one s_barrier.  16-byte chunk c of row r sits at chunk
-// c ^ ((r >> 1) & 7), which makes both the DMA writes (8 lanes per row) and the
-// fragment reads (16 consecutive rows, one chunk) touch 16 distinct 16-byte
+// K advances in 64-element tiles.  A tile is two 32 KB units, its 256 token
+// rows and its 256 weight rows, and LDS is a ring of five such units filled by
+// direct global->LDS loads (global_load_lds_dwordx4, issued from inline assembly
+// so that no compiler-inserted wait serialises them).  While tile kt is being
+// multiplied, the weight unit of tile kt+1..kt+2 and the token unit of tile
+// kt+2..kt+3 are in flight (up to 96 KB per CU: the loop is bound by how many
+// bytes the CU keeps in flight towards L2, not by MFMA issue), and the only
+// per-tile synchronisation is one wait plus one s_barrier.  16-byte chunk c of
+// row r sits at chunk c ^ ((r >> 1) & 7), which makes both the DMA writes (8
+// lanes per row) and the fragment reads (16 consecutive rows, one chunk) touch
+// 16 distinct 16-byte
 // bank groups.  Token fragments holding only padding slots are skipped and
 // their rows are not loaded.
 // The epilogue rounds the accumulators to the activation dtype, parks the
 // wavefront's 128 x 128 tile in LDS and writes it out with 16-byte stores, the
 // gated activation being applied on the way.
 // ---------------------------------------------------------------------------
-constexpr int kBigBM = 256, kBigBNW = 256, kBigBK = 64, kBigStages = 2;
+constexpr int kBigBM = 256, kBigBNW = 256, kBigBK = 64, kBigUnits = 5;
 constexpr int kBigRowBytes = kBigBK * 2;
-constexpr int kBigStageBytes = (kBigBM + kBigBNW) * kBigRowBytes;
+constexpr int kBigUnitBytes = 256 * kBigRowBytes;  // 256 rows of one operand, one K tile
+constexpr int kBigDmaPerUnit = 8;                  // global_load_lds instructions per thread and unit
 constexpr int kEpiRowBytes = 128 * 2 + 16;   // one token row of a wavefront's tile, padded
 constexpr int kEpiWaveBytes = 128 * kEpiRowBytes;
-constexpr int kBigLdsBytes = 4 * kEpiWaveBytes > kBigStages * kBigStageBytes ? 4 * kEpiWaveBytes
-                                                                              : kBigStages * kBigStageBytes;
-
-constexpr int kBigSideBytes = 2 * kBigBM * 4;  // per-slot token id and routed weight, kept for the epilogue
-constexpr int kBigLdsTotal = kBigLdsBytes + kBigSideBytes;
+constexpr int kBigLdsBytes = 4 * kEpiWaveBytes;    // epilogue staging, reuses the ring
+constexpr int kBigSideBytes = 2 * kBigBM * 4;      // per-slot token id and routed weight for the epilogue
+constexpr int kBigLdsTotal = kBigUnits * kBigUnitBytes;  // the whole 160 KB of the CU
+static_assert(kBigLdsBytes + kBigSideBytes + 16 <= kBigLdsTotal, "epilogue staging must fit in the ring");
 
 typedef __attribute__((address_space(3))) char lds_char;
 
@@ -343,14 +347,6 @@ __device__ __forceinline__ void lds_dma16(const char* base, uint32_t lane_byte_o
       :
       : "s"(lds_wave_base), "v"(lane_byte_offset), "s"(base)
       : "memory");
-}
-
-// Touches one dword of a line that a later tile will need, so that the line is
-// in L2 by the time the LDS DMA asks for it.  The value lands in `sink`, which
-// is threaded through every call and read once after the loop, so the register
-// stays reserved while such loads are in flight.
-__device__ __forceinline__ void l2_touch(const char* base, uint32_t lane_byte_offset, uint32_t& sink) {
-  asm volatile("global_load_dword %0, %1, %2" : "+v"(sink) : "v"(lane_byte_offset), "s"(base) : "memory");
 }
 
 template <int N>
@@ -391,45 +387,47 @@ struct BigCtx {
   const char* w_base;   // wave-uniform base of this expert's weights
   uint32_t a_off[8];    // per-lane byte offsets of the eight 32-row load groups
   uint32_t w_off[8];
-  uint32_t dma_lds;     // LDS offset of this wavefront's DMA window in stage 0, group 0
-  int a_groups;         // 32-row token groups that hold real slots
-  uint32_t pf_a_off;    // per-lane byte offset of token row `tid` (L2 prefetch)
-  uint32_t pf_w_off;    // per-lane byte offset of weight row `tid`
-  bool pf_a_live;       // token row `tid` holds a real slot
+  uint32_t dma_lds;     // LDS offset of this wavefront's DMA window in unit slot 0, group 0
   int rd_k[4];          // fragment read offsets for the four MFMA steps of a K tile
-  int x_row;            // byte offset of this wavefront's first token row in a stage
-  int w_row[4];         // byte offsets of this wavefront's weight fragments in a stage
+  int x_row;            // byte offset of this wavefront's first token row in a token unit
+  int w_row[4];         // byte offsets of this wavefront's weight fragments in a weight unit
 };
 
 // Main loop for a wavefront that has FMC live token fragments (0..4).
+// Unit j of the stream  A(0) W(0) A(1) W(1) ...  lives in ring slot j % 5.
 // One K tile is four MFMA steps; two register sets of fragments (P, Q)
 // alternate so that the LDS reads of a step are in flight behind the MFMAs of
 // the previous one:
 //   Q<-(kt,1) mma P | P<-(kt,2) mma Q | Q<-(kt,3) mma P |
-//   wait, barrier, request tile kt+2, P<-(kt+1,0) | mma Q
+//   wait for tile kt+1, barrier, request W(kt+2) and A(kt+3) into the two slots
+//   tile kt just left, P<-(kt+1,0) | mma Q
+// At the wait only A(kt+2), the youngest request, may still be outstanding.
 // sched_barrier keeps the compiler from re-serialising reads and MFMAs.
 template <typename Mma, int FMC>
 __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, int nk,
                                              f32x16 (&acc)[4][4]) {
-  auto issue_tile = [&](int kt) {
-    const uint32_t dst = c.dma_lds + (kt & 1) * kBigStageBytes;
+  auto issue_a = [&](int kt, int slot) {
+    const uint32_t dst = c.dma_lds + slot * kBigUnitBytes;
     const char* ab = c.a_base + kt * kBigRowBytes;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) lds_dma16(ab, c.a_off[i], dst + i * 4096);
+  };
+  auto issue_w = [&](int kt, int slot) {
+    const uint32_t dst = c.dma_lds + slot * kBigUnitBytes;
     const char* wb = c.w_base + kt * kBigRowBytes;
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-      if (i < c.a_groups) lds_dma16(ab, c.a_off[i], dst + i * 4096);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) lds_dma16(wb, c.w_off[i], dst + (8 + i) * 4096);
+    for (int i = 0; i < 8; ++i) lds_dma16(wb, c.w_off[i], dst + i * 4096);
   };
   constexpr int XF = FMC > 0 ? FMC : 1;
-  auto read_frags = [&](int kt, int kk, uint4 (&wf)[4], uint4 (&xf)[XF]) {
+  auto read_frags = [&](int sa, int sw, int kk, uint4 (&wf)[4], uint4 (&xf)[XF]) {
     if constexpr (FMC > 0) {
-      const char* st = smem + (kt & 1) * kBigStageBytes;
+      const char* stw = smem + sw * kBigUnitBytes + c.rd_k[kk];
+      const char* sta = smem + sa * kBigUnitBytes + c.x_row + c.rd_k[kk];
 #pragma unroll
-      for (int fn = 0; fn < 4; ++fn) wf[fn] = *reinterpret_cast<const uint4*>(st + c.w_row[fn] + c.rd_k[kk]);
+      for (int fn = 0; fn < 4; ++fn) wf[fn] = *reinterpret_cast<const uint4*>(stw + c.w_row[fn]);
 #pragma unroll
       for (int fm = 0; fm < FMC; ++fm)
-        xf[fm] = *reinterpret_cast<const uint4*>(st + c.x_row + fm * 32 * kBigRowBytes + c.rd_k[kk]);
+        xf[fm] = *reinterpret_cast<const uint4*>(sta + fm * 32 * kBigRowBytes);
     }
   };
   auto mma_all = [&](const uint4 (&wf)[4], const uint4 (&xf)[XF]) {
@@ -438,59 +436,57 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
 #pragma unroll
       for (int fn = 0; fn < 4; ++fn) acc[fn][fm] = Mma::mma(wf[fn], xf[fm], acc[fn][fm]);
   };
+  auto next_slot = [](int s) { return s + 2 >= kBigUnits ? s + 2 - kBigUnits : s + 2; };
 
-  // Two L2 touches per thread and K tile, kPfAhead tiles ahead of the DMA (one
-  // token line, one weight line; 256 threads cover the 512 lines of a K tile).
-  // Exactly two are issued each time so that "all but the last two vector
-  // memory operations have returned" always means "the DMA of the next tile is
-  // complete".
-  constexpr int kPfAhead = 2;
-  uint32_t sink = 0;
-  auto touch_tile = [&](int kt) {
-    const int t = kt < nk ? kt : nk - 1;
-    l2_touch(c.a_base + t * kBigRowBytes, c.pf_a_off, sink);
-    l2_touch(c.w_base + t * kBigRowBytes, c.pf_w_off, sink);
-  };
-
-  issue_tile(0);
-  wait_vmcnt<0>();
+  // fill the ring: A(0) W(0) A(1) W(1) A(2), then wait for tile 0 only
+  issue_a(0, 0);
+  issue_w(0, 1);
+  if (1 < nk) { issue_a(1, 2); issue_w(1, 3); }
+  if (2 < nk) issue_a(2, 4);
+  if (2 < nk) wait_vmcnt<3 * kBigDmaPerUnit>();
+  else if (1 < nk) wait_vmcnt<2 * kBigDmaPerUnit>();
+  else wait_vmcnt<0>();
   bare_barrier();
-  if (1 < nk) issue_tile(1);
-  touch_tile(2);
-  touch_tile(3);
+  int sa = 0, sw = 1;  // slots of the tile being multiplied
   uint4 wfP[4], xfP[XF], wfQ[4], xfQ[XF];
-  read_frags(0, 0, wfP, xfP);
+  read_frags(sa, sw, 0, wfP, xfP);
   __builtin_amdgcn_sched_barrier(0);
 
   for (int kt = 0; kt < nk; ++kt) {
-    read_frags(kt, 1, wfQ, xfQ);
+#ifdef MOE_TRACE
+    if ((blockIdx.x == 8 || blockIdx.x == 1024) && (threadIdx.x & 63) == 0 && kt < 64)
+      moe_dbg[8 * 4096 + (blockIdx.x == 8 ? 0 : 256) + (threadIdx.x >> 6) * 64 + kt] = __builtin_amdgcn_s_memrealtime();
+#endif
+    read_frags(sa, sw, 1, wfQ, xfQ);
     __builtin_amdgcn_sched_barrier(0);
     mma_all(wfP, xfP);
     __builtin_amdgcn_sched_barrier(0);
-    read_frags(kt, 2, wfP, xfP);
+    read_frags(sa, sw, 2, wfP, xfP);
     __builtin_amdgcn_sched_barrier(0);
     mma_all(wfQ, xfQ);
     __builtin_amdgcn_sched_barrier(0);
-    read_frags(kt, 3, wfQ, xfQ);
+    read_frags(sa, sw, 3, wfQ, xfQ);
     __builtin_amdgcn_sched_barrier(0);
     mma_all(wfP, xfP);
     __builtin_amdgcn_sched_barrier(0);
     if (kt + 1 < nk) {
-      // tile kt+1 has landed (everything but the two newest touches has
-      // returned) and nobody reads stage kt any more (the reads of step 3 have
-      // returned: lgkmcnt(0)) -> it can take tile kt+2
-      asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
+      // tile kt+1 must have landed (only A(kt+2) may still be outstanding) and
+      // nobody reads the slots of tile kt any more (its last fragment reads
+      // have returned: lgkmcnt(0))
+      if (kt + 2 < nk) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       bare_barrier();
-      if (kt + 2 < nk) issue_tile(kt + 2);
-      touch_tile(kt + 2 + kPfAhead);
-      read_frags(kt + 1, 0, wfP, xfP);
+      if (kt + 2 < nk) issue_w(kt + 2, sa);
+      if (kt + 3 < nk) issue_a(kt + 3, sw);
+      sa = next_slot(sa);
+      sw = next_slot(sw);
+      read_frags(sa, sw, 0, wfP, xfP);
     }
     __builtin_amdgcn_sched_barrier(0);
     mma_all(wfQ, xfQ);
     __builtin_amdgcn_sched_barrier(0);
   }
   wait_vmcnt<0>();
-  asm volatile("" ::"v"(sink));
 }
 
 // Epilogue phase 1: round this wavefront's accumulators to the activation dtype
@@ -543,69 +539,87 @@ __device__ __forceinline__ void big_park(const GemmParams& p, int e, int n0, int
 // Epilogue phase 2: write the parked tile to global memory, 8 columns (16 bytes)
 // per lane and step.  Gated: columns [0,64) of a row are gate values, [64,128)
 // the matching up values.
-template <typename El, bool GATED>
+template <typename El>
+__device__ __forceinline__ float unpack_lo(uint32_t w);
+template <typename El>
+__device__ __forceinline__ float unpack_hi(uint32_t w);
+template <>
+__device__ __forceinline__ float unpack_lo<ElemBF16>(uint32_t w) { return __uint_as_float(w << 16); }
+template <>
+__device__ __forceinline__ float unpack_hi<ElemBF16>(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+template <>
+__device__ __forceinline__ float unpack_lo<ElemF16>(uint32_t w) { return f16_bits_to_f32(static_cast<uint16_t>(w)); }
+template <>
+__device__ __forceinline__ float unpack_hi<ElemF16>(uint32_t w) { return f16_bits_to_f32(static_cast<uint16_t>(w >> 16)); }
+
+template <typename El, int ACT>
+__device__ __forceinline__ uint32_t gated_pair(const GemmParams& p, uint32_t gw, uint32_t uw) {
+  const float g0 = unpack_lo<El>(gw), g1 = unpack_hi<El>(gw);
+  const float u0 = unpack_lo<El>(uw), u1 = unpack_hi<El>(uw);
+  if constexpr (ACT == MOE_ACT_SWIGLUOAI) {
+    return pack2<El>(moe_swigluoai(g0, u0, p.alpha, p.limit), moe_swigluoai(g1, u1, p.alpha, p.limit));
+  } else {
+    float a0, a1;
+    if constexpr (ACT == MOE_ACT_SILU) {
+      a0 = silu_fast(g0);
+      a1 = silu_fast(g1);
+    } else {
+      a0 = 0.5f * g0 * (1.f + erff(g0 * 0.70710678118654752f));
+      a1 = 0.5f * g1 * (1.f + erff(g1 * 0.70710678118654752f));
+    }
+    const uint32_t aw = pack2<El>(a0, a1);  // the activation is stored in T before the product
+    return pack2<El>(unpack_lo<El>(aw) * u0, unpack_hi<El>(aw) * u1);
+  }
+}
+
+template <typename El, bool GATED, int ACT>
 __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, int lane, int slot0,
                                           int rows, const int* s_tok, const char* epi) {
   using S = typename El::S;
   constexpr int COLS = GATED ? 64 : 128;      // output columns of the wavefront tile
   constexpr int LPR = COLS / 8;               // lanes per row
   constexpr int RPS = kWave / LPR;            // rows per step
+  constexpr int UNR = 4;                      // steps in flight: LDS reads, math and stores overlap
   const int c8 = (lane % LPR) * 8;
   const int ncol = n0 + wn * COLS + c8;
-  for (int r0 = 0; r0 < rows; r0 += RPS) {
-    const int r = r0 + lane / LPR;
-    if (r >= rows) continue;
-    const int slot = slot0 + r;
-    const int tok = s_tok[r];
-    if (tok >= p.numel) continue;
-    const char* row = epi + r * kEpiRowBytes;
-    uint4 out;
-    if constexpr (GATED) {
-      const uint4 gq = *reinterpret_cast<const uint4*>(row + c8 * 2);
-      const uint4 uq = *reinterpret_cast<const uint4*>(row + (64 + c8) * 2);
-      const uint32_t gw[4] = {gq.x, gq.y, gq.z, gq.w}, uw[4] = {uq.x, uq.y, uq.z, uq.w};
-      uint32_t ow[4];
+  const bool vec_ok = ncol + 7 < p.N && (p.ldc & 7) == 0;
+  for (int r0 = 0; r0 < rows; r0 += RPS * UNR) {
+    int tok[UNR];
+    uint4 gq[UNR], uq[UNR];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float res[2];
-#pragma unroll
-        for (int hlf = 0; hlf < 2; ++hlf) {
-          const float gv = El::ld(static_cast<S>(gw[i] >> (16 * hlf)));
-          const float uv = El::ld(static_cast<S>(uw[i] >> (16 * hlf)));
-          float rr;
-          if (p.activation == MOE_ACT_SILU) {
-            rr = El::ld(El::st(silu_fast(gv))) * uv;
-          } else if (p.activation == MOE_ACT_SWIGLUOAI) {
-            rr = moe_swigluoai(gv, uv, p.alpha, p.limit);
-          } else {
-            const float ge = 0.5f * gv * (1.f + erff(gv * 0.70710678118654752f));
-            rr = El::ld(El::st(ge)) * uv;
-          }
-          res[hlf] = rr;
-        }
-        ow[i] = static_cast<uint32_t>(El::st(res[0])) | (static_cast<uint32_t>(El::st(res[1])) << 16);
-      }
-      out = uint4{ow[0], ow[1], ow[2], ow[3]};
-    } else {
-      out = *reinterpret_cast<const uint4*>(row + c8 * 2);
+    for (int u = 0; u < UNR; ++u) {
+      const int r = r0 + u * RPS + lane / LPR;
+      tok[u] = r < rows ? s_tok[r] : p.numel;
+      const char* row = epi + (r < 128 ? r : 127) * kEpiRowBytes;
+      gq[u] = *reinterpret_cast<const uint4*>(row + c8 * 2);
+      if constexpr (GATED) uq[u] = *reinterpret_cast<const uint4*>(row + (64 + c8) * 2);
     }
-    const int64_t crow = p.a_by_slot ? tok : slot;
-    S* dst = static_cast<S*>(p.c) + crow * p.ldc + ncol;
-    if (ncol + 7 < p.N && (p.ldc & 7) == 0) {
-      *reinterpret_cast<uint4*>(dst) = out;
-    } else {
-      const uint32_t w4[4] = {out.x, out.y, out.z, out.w};
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        if (ncol + i < p.N) dst[i] = static_cast<S>(w4[i >> 1] >> (16 * (i & 1)));
+    for (int u = 0; u < UNR; ++u) {
+      if (tok[u] >= p.numel) continue;
+      uint4 out = gq[u];
+      if constexpr (GATED)
+        out = uint4{gated_pair<El, ACT>(p, gq[u].x, uq[u].x), gated_pair<El, ACT>(p, gq[u].y, uq[u].y),
+                    gated_pair<El, ACT>(p, gq[u].z, uq[u].z), gated_pair<El, ACT>(p, gq[u].w, uq[u].w)};
+      const int slot = slot0 + r0 + u * RPS + lane / LPR;
+      const int64_t crow = p.a_by_slot ? tok[u] : slot;
+      S* dst = static_cast<S*>(p.c) + crow * p.ldc + ncol;
+      if (vec_ok) {
+        *reinterpret_cast<uint4*>(dst) = out;
+      } else {
+        const uint32_t w4[4] = {out.x, out.y, out.z, out.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (ncol + i < p.N) dst[i] = static_cast<S>(w4[i >> 1] >> (16 * (i & 1)));
+      }
     }
   }
 }
 
 template <typename Mma, int FMC, bool GATED>
 __device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, char* smem, int nk,
-                                         int e, int n0, int wn, int lane, float my_rw, float* s_rw_all,
-                                         const float* s_rw, char* epi) {
+                                         int e, int n0, int wn, int lane, int my_tok, float my_rw,
+                                         int* s_tok_all, float* s_rw_all, const float* s_rw, char* epi) {
   using El = typename Mma::El;
   f32x16 acc[4][4];
 #pragma unroll
@@ -615,9 +629,11 @@ __device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, c
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[fn][fm][r] = 0.f;
   big_mainloop<Mma, FMC>(c, smem, nk, acc);
+  bare_barrier();  // every wavefront is done reading the ring before it is reused
+  s_tok_all[threadIdx.x] = my_tok;
   s_rw_all[threadIdx.x] = my_rw;  // requested before the main loop, needed only now
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  bare_barrier();  // every wavefront is done reading the stages before they are reused
+  bare_barrier();
   if constexpr (FMC > 0) big_park<El, FMC, GATED>(p, e, n0, wn, lane >> 5, lane & 31, s_rw, epi, acc);
 }
 
@@ -640,6 +656,7 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   const int l32 = lane & 31, lhi = lane >> 5;
   const int wm = wave & 1, wn = wave >> 1;
   [[maybe_unused]] const unsigned long long t_start = MOE_TRACE_NOW();
+  [[maybe_unused]] const unsigned long long c_start = __builtin_readcyclecounter();
   // the three loads below do not depend on each other: one memory latency, not three
   const int npp = *p.num_post_pad;
   const int e = p.expert_ids[(mb * kBigBM) / p.align_bs];
@@ -650,8 +667,12 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   int* s_tok = reinterpret_cast<int*>(smem + kBigLdsBytes);
   float* s_rw_all = reinterpret_cast<float*>(smem + kBigLdsBytes + kBigBM * 4);
   s_tok[tid] = my_tok;
-  // real slots come first in a block
-  const int nvalid = __syncthreads_count(my_tok < p.numel);
+  // real slots come first in a block: count them (dynamic LDS only, the ring needs all 160 KB)
+  int* s_cnt = reinterpret_cast<int*>(smem + kBigLdsBytes + kBigSideBytes);
+  const int wave_cnt = __popcll(__ballot(my_tok < p.numel));
+  if (lane == 0) s_cnt[wave] = wave_cnt;
+  __syncthreads();
+  const int nvalid = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
   if (nvalid == 0) return;
   float my_rw = 1.f;
   if (p.mul_weight) my_rw = my_tok < p.numel ? p.topk_w[my_tok] : 0.f;
@@ -661,32 +682,16 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   const int ld_chunk = (tid & 7) ^ ((tid >> 4) & 7);  // logical chunk this lane fetches
   c.a_base = static_cast<const char*>(p.a);
   c.w_base = static_cast<const char*>(p.w) + static_cast<int64_t>(e) * p.w_stride_e * 2;
-  c.a_groups = (nvalid + 31) >> 5;
-  {
-    // L2 prefetch: this thread owns token row `tid` and weight row `tid` of the tile
-    const int tok = my_tok;
-    const int64_t src = p.a_by_slot ? static_cast<int64_t>(mb * kBigBM + tid)
-                                    : (tok < p.numel ? tok / p.top_k : 0);
-    c.pf_a_off = static_cast<uint32_t>(src * p.lda * 2);
-    c.pf_a_live = tok < p.numel;
-    int64_t wrow;
-    if constexpr (GATED) {
-      const int half = tid >> 7;
-      int n = n0 + (tid & 127);
-      n = n < p.N ? n : p.N - 1;
-      wrow = p.interleaved ? (2 * n + half) : (half * p.N + n);
-    } else {
-      const int n = n0 + tid;
-      wrow = n < p.N ? n : p.N - 1;
-    }
-    c.pf_w_off = static_cast<uint32_t>(wrow * p.w_stride_n * 2);
-  }
+  const int a_groups = (nvalid + 31) >> 5;  // 32-row token groups that hold real slots
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const int slot = mb * kBigBM + ld_row + 32 * i;
+    // groups made of padding only re-request group 0 (an L1 hit) so that every
+    // token unit is exactly eight loads and the vmcnt bookkeeping stays fixed
+    const int gi = i < a_groups ? i : 0;
+    const int slot = mb * kBigBM + ld_row + 32 * gi;
     int64_t src = slot;
     if (!p.a_by_slot) {
-      const int tok = s_tok[ld_row + 32 * i];
+      const int tok = s_tok[ld_row + 32 * gi];
       src = tok < p.numel ? tok / p.top_k : 0;
     }
     c.a_off[i] = static_cast<uint32_t>((src * p.lda + ld_chunk * 8) * 2);
@@ -714,27 +719,39 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
       r = (fn < 2) ? wn * 64 + fn * 32 : 128 + wn * 64 + (fn - 2) * 32;
     else
       r = wn * 128 + fn * 32;
-    c.w_row[fn] = (kBigBM + r) * kBigRowBytes;
+    c.w_row[fn] = r * kBigRowBytes;
   }
   const int nk = p.Kd / kBigBK;
   const int slot0 = mb * kBigBM + wm * 128;
   char* epi = smem + wave * kEpiWaveBytes;
   [[maybe_unused]] const unsigned long long t_pro = MOE_TRACE_NOW();
   const int rows = min(128, max(0, nvalid - wm * 128));  // real slots of this wavefront
+  __syncthreads();  // s_tok sits inside the ring: everyone has read it before any DMA may land there
   switch ((rows + 31) >> 5) {
-    case 0: big_wave<Mma, 0, GATED>(p, c, smem, nk, e, n0, wn, lane, my_rw, s_rw_all, s_rw_all + wm * 128, epi); break;
-    case 1: big_wave<Mma, 1, GATED>(p, c, smem, nk, e, n0, wn, lane, my_rw, s_rw_all, s_rw_all + wm * 128, epi); break;
-    case 2: big_wave<Mma, 2, GATED>(p, c, smem, nk, e, n0, wn, lane, my_rw, s_rw_all, s_rw_all + wm * 128, epi); break;
-    case 3: big_wave<Mma, 3, GATED>(p, c, smem, nk, e, n0, wn, lane, my_rw, s_rw_all, s_rw_all + wm * 128, epi); break;
-    default: big_wave<Mma, 4, GATED>(p, c, smem, nk, e, n0, wn, lane, my_rw, s_rw_all, s_rw_all + wm * 128, epi); break;
+    case 0: big_wave<Mma, 0, GATED>(p, c, smem, nk, e, n0, wn, lane, my_tok, my_rw, s_tok, s_rw_all, s_rw_all + wm * 128, epi); break;
+    case 1: big_wave<Mma, 1, GATED>(p, c, smem, nk, e, n0, wn, lane, my_tok, my_rw, s_tok, s_rw_all, s_rw_all + wm * 128, epi); break;
+    case 2: big_wave<Mma, 2, GATED>(p, c, smem, nk, e, n0, wn, lane, my_tok, my_rw, s_tok, s_rw_all, s_rw_all + wm * 128, epi); break;
+    case 3: big_wave<Mma, 3, GATED>(p, c, smem, nk, e, n0, wn, lane, my_tok, my_rw, s_tok, s_rw_all, s_rw_all + wm * 128, epi); break;
+    default: big_wave<Mma, 4, GATED>(p, c, smem, nk, e, n0, wn, lane, my_tok, my_rw, s_tok, s_rw_all, s_rw_all + wm * 128, epi); break;
   }
   [[maybe_unused]] const unsigned long long t_main = MOE_TRACE_NOW();
-  big_flush<El, GATED>(p, n0, wn, lane, slot0, rows, s_tok + wm * 128, epi);
+  if constexpr (GATED) {
+    // one tight loop per activation instead of a three-way branch per element
+    if (p.activation == MOE_ACT_SILU)
+      big_flush<El, true, MOE_ACT_SILU>(p, n0, wn, lane, slot0, rows, s_tok + wm * 128, epi);
+    else if (p.activation == MOE_ACT_SWIGLUOAI)
+      big_flush<El, true, MOE_ACT_SWIGLUOAI>(p, n0, wn, lane, slot0, rows, s_tok + wm * 128, epi);
+    else
+      big_flush<El, true, MOE_ACT_GELU>(p, n0, wn, lane, slot0, rows, s_tok + wm * 128, epi);
+  } else {
+    big_flush<El, false, MOE_ACT_SILU>(p, n0, wn, lane, slot0, rows, s_tok + wm * 128, epi);
+  }
 #ifdef MOE_TRACE
   const unsigned long long t_end = MOE_TRACE_NOW();
   if (tid == 0 && blockIdx.x < 4096) {
     moe_dbg[blockIdx.x * 8 + 0] = t_start; moe_dbg[blockIdx.x * 8 + 1] = t_pro;
     moe_dbg[blockIdx.x * 8 + 2] = t_main; moe_dbg[blockIdx.x * 8 + 3] = t_end;
+    moe_dbg[blockIdx.x * 8 + 6] = __builtin_readcyclecounter() - c_start;
     moe_dbg[blockIdx.x * 8 + 4] = nvalid; moe_dbg[blockIdx.x * 8 + 5] = __builtin_amdgcn_s_getreg((20) | (0 << 6) | (3 << 11));
   }
 #endif
