@@ -198,6 +198,7 @@ def main() -> int:
     ap.add_argument("--chunk-mode", default="both", choices=["both", "chunked", "single", "off"],
                     help="config 4 (chunk amplification) leg: both sides, one side only (for "
                          "rocprofv3 counter runs), or off")
+    ap.add_argument("--no-fp8", action="store_true", help="skip the e4m3 leg (config 5)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device copies, the known-size kernel that "
                          "FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -279,6 +280,30 @@ def main() -> int:
 
     if compute_bound and a.chunk_mode != "off":
         out["chunk_amplification"] = chunk_amplification(moe, main_layer, max(2, a.steps // 10), a.chunk_mode)
+    if compute_bound and not a.no_fp8:
+        # config 5: e4m3 weights (per-output-channel scales), per-token e4m3 activations
+        w13q, w13s, w2q, w2s = moe.quantize_expert_weights(main_layer.w13, main_layer.w2)
+
+        def fp8_step():
+            tw, ids8, _ = moe.fused_topk(main_layer.x, main_layer.logits, shape.top_k, True)
+            return moe.fused_experts(main_layer.x, w13q, w2q, None, None, tw, ids8,
+                                     per_channel_quant=True, w1_scale=w13s, w2_scale=w2s)
+
+        for _ in range(a.warmup):
+            fp8_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(a.steps):
+            fp8_step()
+        torch.cuda.synchronize()
+        fms = (time.perf_counter() - t0) * 1e3 / a.steps
+        out["fp8_e4m3"] = {"workload": a.workload, "ms_per_step": round(fms, 4),
+                           "tflops": round(flops / (fms * 1e-3) / 1e12, 2),
+                           "frac_of_fp8_peak": round(flops / (fms * 1e-3) / 1e12 / 5000.0, 4),
+                           "block_size_m": moe.try_get_optimal_moe_config(
+                               main_layer.w13.shape, main_layer.w2.shape, shape.top_k, "fp8_w8a8",
+                               main_layer.T)["BLOCK_SIZE_M"]}
+        del w13q, w2q
     if compute_bound:
         dec = Layer(moe, "decode_256", dev)
         dms = time_steps(dec, max(a.steps, 50), max(a.warmup, 10))

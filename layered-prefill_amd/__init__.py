@@ -13,5 +13,6 @@ CPU or PyTorch fallback.
 """
 from . import _lib, ops, fused_moe, layer, workloads  # noqa: F401
 from .fused_moe import (fused_experts, fused_experts_impl, fused_topk,  # noqa: F401
-                        moe_align_block_size, try_get_optimal_moe_config)
+                        moe_align_block_size, quantize_expert_weights,
+                        try_get_optimal_moe_config)
 from .layer import FusedMoE, FusedMoEParallelConfig, MoEConfig, UnquantizedFusedMoEMethod  # noqa: F401

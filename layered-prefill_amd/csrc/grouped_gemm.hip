@@ -35,6 +35,7 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 struct MmaBF16 {
   using El = ElemBF16;
+  static constexpr int kEs = 2;  // bytes per input element
   static __device__ __forceinline__ f32x16 mma(const uint4& a, const uint4& b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
@@ -42,9 +43,27 @@ struct MmaBF16 {
 };
 struct MmaF16 {
   using El = ElemF16;
+  static constexpr int kEs = 2;
   static __device__ __forceinline__ f32x16 mma(const uint4& a, const uint4& b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+
+// e4m3 (OCP) inputs, one byte per element: a 16-byte chunk holds 16 K elements,
+// i.e. the per-lane operands of two v_mfma_f32_32x32x16_fp8_fp8 steps.  OutEl is
+// the dtype results are rounded to and stored in.
+template <typename OutEl>
+struct MmaE4M3 {
+  using El = OutEl;
+  static constexpr int kEs = 1;
+  static __device__ __forceinline__ f32x16 mma(const uint4& a, const uint4& b, f32x16 c) {
+    const long a0 = static_cast<long>(a.x) | (static_cast<long>(a.y) << 32);
+    const long a1 = static_cast<long>(a.z) | (static_cast<long>(a.w) << 32);
+    const long b0 = static_cast<long>(b.x) | (static_cast<long>(b.y) << 32);
+    const long b1 = static_cast<long>(b.z) | (static_cast<long>(b.w) << 32);
+    c = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a0, b0, c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a1, b1, c, 0, 0, 0);
   }
 };
 
@@ -54,6 +73,9 @@ struct GemmParams {
   void* c;              // pass 1: inter [sorted_cap, ldc]; pass 2: c3 [T*K, ldc]
   const void* bias;     // [E, rows] in the activation dtype, or null
   const float* topk_w;  // [T*K]
+  const float* a_scale; // fp8 only: per-row scale of the A operand (indexed like the A rows)
+  const float* w_scale; // fp8 only: per-weight-row scale, [E, rows]
+  int64_t w_scale_stride_e;
   const int32_t* sorted_ids;
   const int32_t* expert_ids;
   const int32_t* num_post_pad;
@@ -96,6 +118,9 @@ __device__ __forceinline__ void store_fragment(const GemmParams& p, int e, const
   using S = typename El::S;
   const S* bias = static_cast<const S*>(p.bias);
   const float rw = p.mul_weight ? p.topk_w[tok] : 1.f;
+  // fp8: the accumulator is in units of (activation scale x weight scale)
+  const float as = p.a_scale ? p.a_scale[p.a_by_slot ? slot : tok / p.top_k] : 1.f;
+  const float* ws = p.w_scale ? p.w_scale + e * p.w_scale_stride_e : nullptr;
   const int64_t crow = p.a_by_slot ? tok : slot;  // pass 2 writes by token, pass 1 by slot
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
@@ -106,6 +131,10 @@ __device__ __forceinline__ void store_fragment(const GemmParams& p, int e, const
       const int col = (n + i < p.N) ? n + i : p.N - 1;
       if constexpr (GATED) {
         float gv = ga[4 * g + i], uv = ua[4 * g + i];
+        if (ws) {
+          gv *= as * ws[p.interleaved ? 2 * col : col];
+          uv *= as * ws[p.interleaved ? 2 * col + 1 : p.N + col];
+        }
         if (bias) {
           const int64_t grow = p.interleaved ? 2 * col : col;
           const int64_t urow = p.interleaved ? 2 * col + 1 : p.N + col;
@@ -127,6 +156,7 @@ __device__ __forceinline__ void store_fragment(const GemmParams& p, int e, const
         o[i] = El::st(r);
       } else {
         float v = ga[4 * g + i];
+        if (ws) v *= as * ws[col];
         if (bias) v += El::ld(bias[e * p.bias_stride_e + col]);
         o[i] = El::st(v * rw);
       }
@@ -146,6 +176,9 @@ __device__ __forceinline__ void store_fragment(const GemmParams& p, int e, const
 template <typename Mma, int BM, int BNW, int WAVES_M, bool GATED>
 __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams p) {
   using El = typename Mma::El;
+  constexpr int ES = Mma::kEs;               // bytes per input element
+  constexpr int BKE = kRowBytes / ES;        // K elements per staged 128-byte row
+  constexpr int CE = 16 / ES;                // K elements per 16-byte chunk
   constexpr int WAVES_N = 4 / WAVES_M;
   constexpr int TM = BM / WAVES_M, FM = TM / 32;     // token fragments per wavefront
   constexpr int TNW = BNW / WAVES_N, FN = TNW / 32;  // weight-row fragments per wavefront
@@ -187,7 +220,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
       const int tok = p.sorted_ids[slot];
       src = tok < p.numel ? tok / p.top_k : 0;
     }
-    a_src[j] = static_cast<const char*>(p.a) + (src * p.lda + ld_c * 8) * 2;
+    a_src[j] = static_cast<const char*>(p.a) + (src * p.lda + ld_c * CE) * ES;
   }
   const char* w_src[B_LD];
 #pragma unroll
@@ -204,7 +237,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
       wrow = n < p.N ? n : p.N - 1;
     }
     w_src[j] = static_cast<const char*>(p.w) +
-               (static_cast<int64_t>(e) * p.w_stride_e + wrow * p.w_stride_n + ld_c * 8) * 2;
+               (static_cast<int64_t>(e) * p.w_stride_e + wrow * p.w_stride_n + ld_c * CE) * ES;
   }
   const int st_off = swizzled(ld_row, ld_c);  // rows 32 apart share the swizzle
 
@@ -235,10 +268,10 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
       for (int r = 0; r < 16; ++r) acc[fn][fm][r] = 0.f;
 
   uint4 a_reg[A_LD], b_reg[B_LD];
-  const int nk = (p.Kd + kBK - 1) / kBK;
+  const int nk = (p.Kd + BKE - 1) / BKE;
 
   auto gload = [&](int kt) {
-    const bool in_k = kt * kBK + ld_c * 8 < p.Kd;
+    const bool in_k = kt * BKE + ld_c * CE < p.Kd;
 #pragma unroll
     for (int j = 0; j < A_LD; ++j)
       a_reg[j] = in_k ? *reinterpret_cast<const uint4*>(a_src[j] + kt * kRowBytes) : uint4{0, 0, 0, 0};
@@ -803,7 +836,9 @@ int launch(const GemmParams& p, hipStream_t s) {
 template <typename Mma, bool GATED>
 int launch_bm(GemmParams& p, int block_size, int64_t sorted_cap, hipStream_t s) {
   p.align_bs = block_size;
-  if (block_size % 256 == 0 && p.Kd % kBigBK == 0) return launch_big<Mma, GATED>(p, sorted_cap, s);
+  if constexpr (Mma::kEs == 2) {
+    if (block_size % 256 == 0 && p.Kd % kBigBK == 0) return launch_big<Mma, GATED>(p, sorted_cap, s);
+  }
   if (block_size % 128 == 0) {
     p.num_m_blocks = static_cast<int>((sorted_cap + 127) / 128);
     p.num_n_tiles = (p.N + (GATED ? 64 : 128) - 1) / (GATED ? 64 : 128);
@@ -828,10 +863,9 @@ int elem_size(int dtype) { return dtype == MOE_F32 ? 4 : (dtype == MOE_E4M3 ? 1 
 
 MOE_EXPORT int moe_preferred_block_size(int M, int E, int K, int act_dtype, int weight_dtype) {
   (void)act_dtype;
-  (void)weight_dtype;
   if (E < 1) return 64;
   const int64_t avg = static_cast<int64_t>(M) * K / E;  // routed rows per expert
-  if (avg >= 256) return 256;
+  if (avg >= 256 && weight_dtype != MOE_E4M3) return 256;  // no large-tile e4m3 kernel yet
   if (avg >= 96) return 128;
   if (avg >= 24) return 64;
   return 32;
@@ -840,13 +874,16 @@ MOE_EXPORT int moe_preferred_block_size(int M, int E, int K, int act_dtype, int 
 MOE_EXPORT int64_t moe_fused_experts_workspace_bytes(int T, int H, int I, int E, int K,
                                                      int block_size, int act_dtype,
                                                      int weight_dtype) {
-  (void)weight_dtype;
   if (T < 0 || H < 1 || I < 1 || E < 1 || K < 1 || block_size < 1) return 0;
   const int64_t numel = static_cast<int64_t>(T) * K;
   const int64_t sorted_cap = numel + static_cast<int64_t>(E) * (block_size - 1);
   const int64_t rows = moe_align_up(sorted_cap, block_size);
   const int64_t es = elem_size(act_dtype);
-  return moe_align_up(rows * I * es, 256) + moe_align_up(numel * H * es, 256);
+  int64_t bytes = moe_align_up(rows * I * es, 256) + moe_align_up(numel * H * es, 256);
+  if (weight_dtype == MOE_E4M3)  // e4m3 copies of x and of the intermediate, one fp32 scale per row
+    bytes += moe_align_up(static_cast<int64_t>(T) * H, 256) + moe_align_up(static_cast<int64_t>(T) * 4, 256) +
+             moe_align_up(rows * I, 256) + moe_align_up(rows * 4, 256);
+  return bytes;
 }
 
 MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
@@ -859,8 +896,13 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
     return moe_fail(MOE_ERR_ARG, "fused_experts: null tensor pointer");
   if (a->act_dtype != MOE_BF16 && a->act_dtype != MOE_F16)
     return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: activation dtype code %d (bf16 and fp16 are built)", a->act_dtype);
-  if (a->weight_dtype != a->act_dtype)
+  const bool fp8 = a->weight_dtype == MOE_E4M3;
+  if (!fp8 && a->weight_dtype != a->act_dtype)
     return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: weight dtype code %d with activation dtype code %d", a->weight_dtype, a->act_dtype);
+  if (fp8 && (!a->w13_scale || !a->w2_scale))
+    return moe_fail(MOE_ERR_ARG, "fused_experts: e4m3 weights need w13_scale and w2_scale");
+  if (fp8 && (a->H % 16 || a->I % 16 || a->w13_stride_n % 16 || a->w2_stride_n % 16 || a->w13_stride_e % 16 || a->w2_stride_e % 16))
+    return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: e4m3 path needs H, I and weight strides in multiples of 16");
   if (a->activation < MOE_ACT_SILU || a->activation > MOE_ACT_GELU)
     return moe_fail(MOE_ERR_ARG, "fused_experts: unknown activation code %d", a->activation);
   if (a->H % 8 || a->I % 8)
@@ -888,6 +930,10 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   const int64_t rows = moe_align_up(a->sorted_cap, a->block_size);
   char* inter = static_cast<char*>(a->workspace);
   char* c3 = inter + moe_align_up(rows * a->I * es, 256);
+  char* xq = c3 + moe_align_up(numel * a->H * es, 256);                        // fp8 only from here on
+  float* xs = reinterpret_cast<float*>(xq + moe_align_up(static_cast<int64_t>(a->T) * a->H, 256));
+  char* iq = reinterpret_cast<char*>(xs) + moe_align_up(static_cast<int64_t>(a->T) * 4, 256);
+  float* is = reinterpret_cast<float*>(iq + moe_align_up(rows * a->I, 256));
 
   GemmParams p{};
   p.sorted_ids = a->sorted_token_ids;
@@ -912,9 +958,17 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.mul_weight = a->apply_router_weight_on_input ? 1 : 0;
   const int passes = a->passes ? a->passes : 7;
   int rc = MOE_OK;
-  if (passes & 1)
+  if (fp8 && (passes & 1)) {
+    // dynamic per-token e4m3 activations: s[t] = amax|x[t]| / 448
+    rc = moe_quant_rows_e4m3(a->x, a->act_dtype, a->T, a->H, reinterpret_cast<uint8_t*>(xq), xs, a->stream);
+    if (rc) return rc;
+    p.a = xq; p.a_scale = xs; p.w_scale = a->w13_scale; p.w_scale_stride_e = 2LL * a->I;
+    rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaE4M3<ElemBF16>, true>(p, a->block_size, a->sorted_cap, s)
+                                  : launch_bm<MmaE4M3<ElemF16>, true>(p, a->block_size, a->sorted_cap, s);
+  } else if (passes & 1) {
     rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaBF16, true>(p, a->block_size, a->sorted_cap, s)
                                   : launch_bm<MmaF16, true>(p, a->block_size, a->sorted_cap, s);
+  }
   if (rc) return rc;
 
   // pass 2: inter . W2^T times the routed weight, rows written by flat token id
@@ -922,9 +976,17 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.bias = a->w2_bias; p.bias_stride_e = a->H;
   p.c = c3; p.ldc = a->H; p.Kd = a->I; p.N = a->H; p.a_by_slot = 1;
   p.mul_weight = a->apply_router_weight_on_input ? 0 : 1;
-  if (passes & 2)
+  if (fp8 && (passes & 2)) {
+    // the activated intermediate is quantised per slot row the same way
+    rc = moe_quant_rows_e4m3(inter, a->act_dtype, rows, a->I, reinterpret_cast<uint8_t*>(iq), is, a->stream);
+    if (rc) return rc;
+    p.a = iq; p.a_scale = is; p.w_scale = a->w2_scale; p.w_scale_stride_e = a->H;
+    rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaE4M3<ElemBF16>, false>(p, a->block_size, a->sorted_cap, s)
+                                  : launch_bm<MmaE4M3<ElemF16>, false>(p, a->block_size, a->sorted_cap, s);
+  } else if (passes & 2) {
     rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaBF16, false>(p, a->block_size, a->sorted_cap, s)
                                   : launch_bm<MmaF16, false>(p, a->block_size, a->sorted_cap, s);
+  }
   if (rc) return rc;
 
   // top-k combine (nanovllm/layers/for_moe/moe_easy_kernel.py:26-31)

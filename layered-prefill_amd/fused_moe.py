@@ -40,8 +40,8 @@ def try_get_optimal_moe_config(w1_shape, w2_shape, top_k: int, dtype: Optional[s
     the only entry that still matters to callers is BLOCK_SIZE_M, the block size
     handed to moe_align_block_size."""
     E = w2_shape[0]
-    bm = lib().moe_preferred_block_size(M, E, top_k, _lib.DTYPE_CODE[torch.bfloat16],
-                                        _lib.DTYPE_CODE[torch.bfloat16])
+    weight_code = _lib.E4M3_CODE if dtype == "fp8_w8a8" else _lib.DTYPE_CODE[torch.bfloat16]
+    bm = lib().moe_preferred_block_size(M, E, top_k, _lib.DTYPE_CODE[torch.bfloat16], weight_code)
     return {"BLOCK_SIZE_M": bm}
 
 
@@ -150,6 +150,16 @@ def launch_fused_experts(x: torch.Tensor, out: torch.Tensor, w1: torch.Tensor, w
         check(L.moe_fused_experts(args))
 
 
+def quantize_expert_weights(w13: torch.Tensor, w2: torch.Tensor):
+    """One-time e4m3 quantisation of expert weights with one scale per output
+    channel, s = amax|row| / 448 (no counterpart in the reference).  Returns
+    (w13_q, w13_scale, w2_q, w2_scale); the quantised tensors are
+    ``torch.float8_e4m3fn`` views."""
+    w13_q, w13_s = ops.quant_rows_e4m3(w13.contiguous())
+    w2_q, w2_s = ops.quant_rows_e4m3(w2.contiguous())
+    return w13_q.view(torch.float8_e4m3fn), w13_s, w2_q.view(torch.float8_e4m3fn), w2_s
+
+
 _FP8_DTYPES = tuple(getattr(torch, n) for n in ("float8_e4m3fn",) if hasattr(torch, n))
 
 
@@ -193,7 +203,17 @@ def fused_experts_impl(hidden_states: torch.Tensor,
 
     fp8 = w1.dtype in _FP8_DTYPES or (w1_scale is not None)
     if fp8:
+        # e4m3 weights with one fp32 scale per output channel (w1_scale [E, 2I], w2_scale
+        # [E, H]); activations are quantised per token inside the call.  The reference
+        # carries these keywords but asserts them None (for_moe/fused_moe.py:248-249).
         assert w1_scale is not None and w2_scale is not None, "fp8 weights need w1_scale and w2_scale"
+        assert w1.dtype in _FP8_DTYPES + (torch.uint8,) and w2.dtype == w1.dtype, \
+            "fp8 weights must be float8_e4m3fn (or its uint8 codes)"
+        assert tuple(w1_scale.shape) == tuple(w1.shape[:2]) and tuple(w2_scale.shape) == tuple(w2.shape[:2]), \
+            "per-output-channel scales expected"
+        assert w1_scale.dtype == torch.float32 and w2_scale.dtype == torch.float32
+        assert w1_scale.is_contiguous() and w2_scale.is_contiguous()
+        assert w1_bias is None and w2_bias is None, "biases are not supported on the fp8 path"
         weight_code = _lib.E4M3_CODE
     else:
         assert w1.dtype == hidden_states.dtype and w2.dtype == hidden_states.dtype, \
@@ -209,7 +229,8 @@ def fused_experts_impl(hidden_states: torch.Tensor,
     top_k_num = topk_ids.size(1)
     CHUNK_SIZE: int = 64 * 1024
     M = min(num_tokens, CHUNK_SIZE)
-    config = try_get_optimal_moe_config(w1.size(), w2.size(), top_k_num, None, M)
+    config_dtype = "fp8_w8a8" if fp8 else None
+    config = try_get_optimal_moe_config(w1.size(), w2.size(), top_k_num, config_dtype, M)
 
     out_hidden_states = hidden_states if inplace else torch.empty_like(hidden_states)
     if topk_weights.dtype != torch.float32:
@@ -228,7 +249,7 @@ def fused_experts_impl(hidden_states: torch.Tensor,
         if tokens_in_chunk <= 0:
             break
         if tokens_in_chunk < CHUNK_SIZE and chunk > 0:
-            config = try_get_optimal_moe_config(w1.size(), w2.size(), top_k_num, None,
+            config = try_get_optimal_moe_config(w1.size(), w2.size(), top_k_num, config_dtype,
                                                 tokens_in_chunk)
         bm = config["BLOCK_SIZE_M"]
         curr_ids = topk_ids[begin:end]

@@ -309,12 +309,20 @@ def fused_experts_ref(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.T
 
 def fused_experts_fp8_ref(hidden_states: torch.Tensor, w1_q: torch.Tensor, w1_scale: torch.Tensor,
                           w2_q: torch.Tensor, w2_scale: torch.Tensor,
-                          topk_weights: torch.Tensor, topk_ids: torch.Tensor) -> torch.Tensor:
+                          topk_weights: torch.Tensor, topk_ids: torch.Tensor,
+                          mirror_rounding: bool = False) -> torch.Tensor:
     """fp32 reference of the fp8 variant (not implemented by the reference:
     nanovllm/layers/for_moe/fused_moe.py:248-249,571,607 assert the scales are
     None): e4m3 per-output-channel weights, dynamic per-token e4m3 activations
-    in front of both GEMMs, everything dequantised and multiplied in fp32."""
-    x = _cpu(hidden_states).float()
+    in front of both GEMMs, everything dequantised and multiplied in fp32.
+
+    ``mirror_rounding=True`` additionally rounds to the activation dtype where
+    the bf16 path stores an intermediate (GEMM1 result, silu, silu*up, weighted
+    GEMM2 result, top-k sum), i.e. the second quantisation sees the stored
+    16-bit intermediate rather than its fp32 value."""
+    x16 = _cpu(hidden_states)
+    dt = x16.dtype if mirror_rounding else None
+    x = x16.float()
     T, H = x.shape
     E, N, _ = w1_q.shape
     K = topk_ids.shape[1]
@@ -322,7 +330,8 @@ def fused_experts_fp8_ref(hidden_states: torch.Tensor, w1_q: torch.Tensor, w1_sc
     tw = _cpu(topk_weights).float()
     xq, xs = quant_act_per_token(x)
     xd = dequant_e4m3(xq) * xs[:, None]
-    out = torch.zeros(T, w2_q.shape[1], dtype=torch.float32)
+    out_k = torch.zeros(T, K, w2_q.shape[1], dtype=torch.float32)
+    w1_q, w2_q = _cpu(w1_q).view(torch.uint8), _cpu(w2_q).view(torch.uint8)
     for e in range(E):
         tok, slot = torch.nonzero(ids == e, as_tuple=True)
         if tok.numel() == 0:
@@ -330,11 +339,13 @@ def fused_experts_fp8_ref(hidden_states: torch.Tensor, w1_q: torch.Tensor, w1_sc
         W1 = dequant_e4m3(w1_q[e]) * _cpu(w1_scale[e]).float()[:, None]
         W2 = dequant_e4m3(w2_q[e]) * _cpu(w2_scale[e]).float()[:, None]
         c1 = xd[tok] @ W1.t()
-        d = N // 2
-        g, u = c1[:, :d], c1[:, d:]
-        c2 = g / (1 + torch.exp(-g)) * u
+        if dt is None:
+            d = N // 2
+            g, u = c1[:, :d], c1[:, d:]
+            c2 = g / (1 + torch.exp(-g)) * u
+        else:
+            c2 = silu_and_mul(c1.to(dt)).float()
         cq, cs = quant_act_per_token(c2)
         c2d = dequant_e4m3(cq) * cs[:, None]
-        c3 = (c2d @ W2.t()) * tw[tok, slot, None]
-        out.index_add_(0, tok, c3)
-    return out
+        out_k[tok, slot] = _round((c2d @ W2.t()) * tw[tok, slot, None], dt)
+    return _round(out_k.sum(dim=1), dt)
