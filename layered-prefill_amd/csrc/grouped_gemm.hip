@@ -50,6 +50,19 @@ struct MmaF16 {
   }
 };
 
+// fp32 inputs through v_mfma_f32_32x32x2_f32: a 16-byte chunk holds four K
+// elements, one per MFMA step (K = 2 per step: one element from each lane half).
+struct MmaF32 {
+  using El = ElemF32;
+  static constexpr int kEs = 4;
+  static __device__ __forceinline__ f32x16 mma(const uint4& a, const uint4& b, f32x16 c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
+  }
+};
+
 // e4m3 (OCP) inputs, one byte per element: a 16-byte chunk holds 16 K elements,
 // i.e. the per-lane operands of two v_mfma_f32_32x32x16_fp8_fp8 steps.  OutEl is
 // the dtype results are rounded to and stored in.
@@ -163,8 +176,12 @@ __device__ __forceinline__ void store_fragment(const GemmParams& p, int e, const
     }
     S* dst = static_cast<S*>(p.c) + crow * p.ldc + n;
     if (n + 3 < p.N && (p.ldc & 3) == 0) {
-      *reinterpret_cast<uint2*>(dst) = uint2{static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16),
-                                             static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16)};
+      if constexpr (sizeof(S) == 4) {
+        *reinterpret_cast<float4*>(dst) = float4{o[0], o[1], o[2], o[3]};
+      } else {
+        *reinterpret_cast<uint2*>(dst) = uint2{static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16),
+                                               static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16)};
+      }
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
@@ -894,8 +911,10 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   if (!a->x || !a->out || !a->w13 || !a->w2 || !a->topk_weights || !a->sorted_token_ids ||
       !a->expert_ids || !a->num_tokens_post_pad)
     return moe_fail(MOE_ERR_ARG, "fused_experts: null tensor pointer");
-  if (a->act_dtype != MOE_BF16 && a->act_dtype != MOE_F16)
-    return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: activation dtype code %d (bf16 and fp16 are built)", a->act_dtype);
+  if (a->act_dtype != MOE_BF16 && a->act_dtype != MOE_F16 && a->act_dtype != MOE_F32)
+    return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: activation dtype code %d", a->act_dtype);
+  if (a->act_dtype == MOE_F32 && a->weight_dtype == MOE_E4M3)
+    return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: e4m3 weights need bf16 or fp16 activations");
   const bool fp8 = a->weight_dtype == MOE_E4M3;
   if (!fp8 && a->weight_dtype != a->act_dtype)
     return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: weight dtype code %d with activation dtype code %d", a->weight_dtype, a->act_dtype);
@@ -966,8 +985,9 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
     rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaE4M3<ElemBF16>, true>(p, a->block_size, a->sorted_cap, s)
                                   : launch_bm<MmaE4M3<ElemF16>, true>(p, a->block_size, a->sorted_cap, s);
   } else if (passes & 1) {
-    rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaBF16, true>(p, a->block_size, a->sorted_cap, s)
-                                  : launch_bm<MmaF16, true>(p, a->block_size, a->sorted_cap, s);
+    rc = a->act_dtype == MOE_BF16  ? launch_bm<MmaBF16, true>(p, a->block_size, a->sorted_cap, s)
+         : a->act_dtype == MOE_F16 ? launch_bm<MmaF16, true>(p, a->block_size, a->sorted_cap, s)
+                                   : launch_bm<MmaF32, true>(p, a->block_size, a->sorted_cap, s);
   }
   if (rc) return rc;
 
@@ -984,8 +1004,9 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
     rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaE4M3<ElemBF16>, false>(p, a->block_size, a->sorted_cap, s)
                                   : launch_bm<MmaE4M3<ElemF16>, false>(p, a->block_size, a->sorted_cap, s);
   } else if (passes & 2) {
-    rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaBF16, false>(p, a->block_size, a->sorted_cap, s)
-                                  : launch_bm<MmaF16, false>(p, a->block_size, a->sorted_cap, s);
+    rc = a->act_dtype == MOE_BF16  ? launch_bm<MmaBF16, false>(p, a->block_size, a->sorted_cap, s)
+         : a->act_dtype == MOE_F16 ? launch_bm<MmaF16, false>(p, a->block_size, a->sorted_cap, s)
+                                   : launch_bm<MmaF32, false>(p, a->block_size, a->sorted_cap, s);
   }
   if (rc) return rc;
 

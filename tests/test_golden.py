@@ -54,8 +54,11 @@ def test_gpu_matches_tiny_fixture(moe, dev):
     s, e, n = moe.moe_align_block_size(ids, 16, shape.experts)
     assert np.array_equal(s.cpu().numpy(), g["sorted_token_ids"])
     assert np.array_equal(e.cpu().numpy(), g["expert_ids"]) and n.item() == g["num_tokens_post_pad"][0]
-    out = moe.fused_experts(x.bfloat16().to(dev), w13.bfloat16().to(dev), w2.bfloat16().to(dev), None, None, tw, ids)
     ref = torch.from_numpy(g["out"])
+    # config 1 as stated (fp32 tensors): only the summation order differs
+    out32 = moe.fused_experts(x.to(dev), w13.to(dev), w2.to(dev), None, None, tw, ids)
+    assert torch.allclose(out32.cpu(), ref, rtol=1e-4, atol=1e-6), (out32.cpu() - ref).abs().max().item()
+    out = moe.fused_experts(x.bfloat16().to(dev), w13.bfloat16().to(dev), w2.bfloat16().to(dev), None, None, tw, ids)
     err = (out.float().cpu() - ref).abs()
     # bf16 inputs and intermediates against the fp32 fixture: rtol 2e-2, atol 1e-2
     assert bool((err <= 1e-2 + 2e-2 * ref.abs()).all()), err.max().item()

@@ -42,6 +42,18 @@ def test_fused_experts_against_oracle(moe, oracle, dev, dtype, E, H, I, T, K):
     _close(out, mirrored, rtol=1.6e-2, atol=2e-3)
 
 
+@pytest.mark.parametrize("E,H,I,T,K", [(8, 256, 128, 64, 2), (16, 512, 192, 300, 4), (3, 72, 40, 50, 2)])
+def test_fused_experts_fp32_against_oracle(moe, oracle, dev, E, H, I, T, K):
+    """fp32 activations and weights (the reference accepts them,
+    nanovllm/layers/for_moe/fused_moe.py:491-493): fp32 MFMA, no rounding points,
+    so only the summation order separates the result from the fp32 oracle."""
+    x, w13, w2, logits = _layer(E, H, I, T, K, 7 + E + T, torch.float32)
+    tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
+    out = moe.fused_experts(x.to(dev), w13.to(dev), w2.to(dev), None, None, tw.to(dev), ids.to(dev))
+    assert out.dtype == torch.float32
+    _close(out, oracle.fused_experts_ref(x, w13, w2, tw, ids), rtol=1e-4, atol=1e-5)
+
+
 @pytest.mark.parametrize("bm", [32, 64, 96, 128, 256, 512])
 def test_every_block_size_kernel(moe, oracle, dev, bm, monkeypatch):
     x, w13, w2, logits = _layer(16, 256, 128, 500, 4, 5, torch.bfloat16)
