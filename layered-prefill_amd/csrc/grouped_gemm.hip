@@ -21,7 +21,7 @@
 
 #ifdef MOE_TRACE
 // Development aid (make EXTRA=-DMOE_TRACE): per-workgroup phase timestamps of the large-tile kernel.
-__device__ unsigned long long moe_dbg[8 * 4096 + 4 * 128];
+__device__ unsigned long long moe_dbg[8 * 4096 + 4 * 128 + 4 * 4096];
 #define MOE_TRACE_NOW() __builtin_amdgcn_s_memrealtime()
 #else
 #define MOE_TRACE_NOW() 0ull
@@ -107,6 +107,8 @@ struct GemmParams {
   float alpha, limit;
   int64_t sorted_cap; // capacity of sorted_ids
   int align_bs;      // block size the alignment was made with (a multiple of the kernel's M tile)
+  int cold_max;      // large-tile kernel: skip alignment blocks with at most this many real slots;
+                     // small-block kernel: when >= 0, take only those blocks (-1: take all)
   int m_major;       // workgroup order inside an XCD: all n-tiles of an m-block are neighbours
 };
 
@@ -209,18 +211,29 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
   // Workgroups are handed to the 8 XCDs round-robin; give each XCD one
   // contiguous range of the (n-tile major, m-block minor) order so that a strip
   // of expert weights is pulled through one L2 only.
-  const int per_xcd = gridDim.x / kXcds;
-  const int logical = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
-  if (logical >= p.num_m_blocks * p.num_n_tiles) return;
+  // The grid covers the worst-case padding; only the m-blocks below the padded
+  // total are live, and the ranges are cut from those so every XCD gets the same share.
+  const int live_mb = (*p.num_post_pad + BM - 1) / BM;
+  const int live = live_mb * p.num_n_tiles;
+  const int per_xcd = (live + kXcds - 1) / kXcds;
+  const int xslot = blockIdx.x / kXcds;
+  const int logical = (blockIdx.x % kXcds) * per_xcd + xslot;
+  if (xslot >= per_xcd || logical >= live) return;
   int nt, mb;
   if (p.m_major) {
     mb = logical / p.num_n_tiles;
     nt = logical - mb * p.num_n_tiles;
   } else {
-    nt = logical / p.num_m_blocks;
-    mb = logical - nt * p.num_m_blocks;
+    nt = logical / live_mb;
+    mb = logical - nt * live_mb;
   }
-  if (mb * BM >= *p.num_post_pad) return;
+  // real slots come first in an alignment block: a tile that starts on padding is empty
+  if (p.sorted_ids[mb * BM] >= p.numel) return;
+  if (p.cold_max >= 0) {
+    // split launch: this kernel only serves alignment blocks with few real slots
+    const int blk0 = (mb * BM) / p.align_bs * p.align_bs;
+    if (p.cold_max < p.align_bs && p.sorted_ids[blk0 + p.cold_max] < p.numel) return;
+  }
   const int e = p.expert_ids[(mb * BM) / p.align_bs];
   const int n0 = nt * BN_OUT;
 
@@ -446,27 +459,31 @@ struct BigCtx {
 // Main loop for a wavefront that has FMC live token fragments (0..4).
 // Unit j of the stream  A(0) W(0) A(1) W(1) ...  lives in ring slot j % 5.
 // One K tile is four MFMA steps; two register sets of fragments (P, Q)
-// alternate so that the LDS reads of a step are in flight behind the MFMAs of
-// the previous one:
-//   Q<-(kt,1) mma P | P<-(kt,2) mma Q | Q<-(kt,3) mma P |
-//   wait for tile kt+1, barrier, request W(kt+2) and A(kt+3) into the two slots
-//   tile kt just left, P<-(kt+1,0) | mma Q
+// alternate, and every step carries, between its MFMAs, the LDS reads of the
+// next step's fragments and four of the sixteen DMA requests of the K tile:
+//   step P(kt,0) reads Q(kt,1), requests W(kt+1)[4..7]
+//   step Q(kt,1) reads P(kt,2), requests A(kt+2)[0..3]
+//   step P(kt,2) reads Q(kt,3), requests A(kt+2)[4..7]
+//   wait for tile kt+1, barrier (frees the two slots of tile kt)
+//   step Q(kt,3) reads P(kt+1,0), requests W(kt+2)[0..3]
 // At the wait only A(kt+2), the youngest request, may still be outstanding.
-// sched_barrier keeps the compiler from re-serialising reads and MFMAs.
+// sched_barrier pins this order against the compiler's scheduler.
 template <typename Mma, int FMC>
 __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, int nk,
                                              f32x16 (&acc)[4][4]) {
+  auto dma_a = [&](int kt, int slot, int i) {
+    lds_dma16(c.a_base + kt * kBigRowBytes, c.a_off[i], c.dma_lds + slot * kBigUnitBytes + i * 4096);
+  };
+  auto dma_w = [&](int kt, int slot, int i) {
+    lds_dma16(c.w_base + kt * kBigRowBytes, c.w_off[i], c.dma_lds + slot * kBigUnitBytes + i * 4096);
+  };
   auto issue_a = [&](int kt, int slot) {
-    const uint32_t dst = c.dma_lds + slot * kBigUnitBytes;
-    const char* ab = c.a_base + kt * kBigRowBytes;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) lds_dma16(ab, c.a_off[i], dst + i * 4096);
+    for (int i = 0; i < 8; ++i) dma_a(kt, slot, i);
   };
   auto issue_w = [&](int kt, int slot) {
-    const uint32_t dst = c.dma_lds + slot * kBigUnitBytes;
-    const char* wb = c.w_base + kt * kBigRowBytes;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) lds_dma16(wb, c.w_off[i], dst + i * 4096);
+    for (int i = 0; i < 8; ++i) dma_w(kt, slot, i);
   };
   constexpr int XF = FMC > 0 ? FMC : 1;
   auto read_frags = [&](int sa, int sw, int kk, uint4 (&wf)[4], uint4 (&xf)[XF]) {
@@ -480,11 +497,42 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
         xf[fm] = *reinterpret_cast<const uint4*>(sta + fm * 32 * kBigRowBytes);
     }
   };
-  auto mma_all = [&](const uint4 (&wf)[4], const uint4 (&xf)[XF]) {
+  // One MFMA step on fragment set X.  The LDS reads of the next step's set Y
+  // and four DMA requests are spread between its MFMAs instead of being issued
+  // back to back: the LDS and the vector memory path each take one wavefront
+  // request every few dozen clocks when all four wavefronts stream, so a burst
+  // stalls the wavefront, and with it the matrix pipe, until the queue drains.
+  // Reads go out in the order the next step consumes them.
+  auto step = [&](const uint4 (&wfX)[4], const uint4 (&xfX)[XF], uint4 (&wfY)[4], uint4 (&xfY)[XF],
+                  bool load_y, int ya, int yw, int ykk, auto&& dma) {
+    const char* stw = smem + yw * kBigUnitBytes + c.rd_k[ykk];
+    const char* sta = smem + ya * kBigUnitBytes + c.x_row + c.rd_k[ykk];
+    auto read_y = [&](int r) {  // r: 0 x0, 1..4 w0..w3, 5.. x1..
+      if constexpr (FMC > 0) {
+        if (!load_y) return;
+        if (r == 0) xfY[0] = *reinterpret_cast<const uint4*>(sta);
+        else if (r <= 4) wfY[r - 1] = *reinterpret_cast<const uint4*>(stw + c.w_row[r - 1]);
+        else if (r - 4 < FMC) xfY[r - 4] = *reinterpret_cast<const uint4*>(sta + (r - 4) * 32 * kBigRowBytes);
+      }
+    };
+    constexpr int NM = 4 * FMC;  // MFMAs of this step
 #pragma unroll
-    for (int fm = 0; fm < FMC; ++fm)
+    for (int m = 0; m < (NM > 0 ? NM : 1); ++m) {
+      if constexpr (NM > 0) {
+        const int fm = m >> 2, fn = m & 3;
+        acc[fn][fm] = Mma::mma(wfX[fn], xfX[fm], acc[fn][fm]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if ((m & 1) == 0) read_y(m >> 1);
+      if ((m & 3) == 3) dma(m >> 2);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // wavefronts with fewer live fragments have fewer MFMAs to hide requests behind
 #pragma unroll
-      for (int fn = 0; fn < 4; ++fn) acc[fn][fm] = Mma::mma(wf[fn], xf[fm], acc[fn][fm]);
+    for (int r = (NM + 1) / 2; r < 8; ++r) read_y(r);
+#pragma unroll
+    for (int i = NM / 4; i < 4; ++i) dma(i);
+    __builtin_amdgcn_sched_barrier(0);
   };
   auto next_slot = [](int s) { return s + 2 >= kBigUnits ? s + 2 - kBigUnits : s + 2; };
 
@@ -498,45 +546,56 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
   else wait_vmcnt<0>();
   bare_barrier();
   int sa = 0, sw = 1;  // slots of the tile being multiplied
+  int fa = 0, fw = 0;  // slots the previous tile left free: W(kt+1) goes to fa, A(kt+2) to fw
   uint4 wfP[4], xfP[XF], wfQ[4], xfQ[XF];
   read_frags(sa, sw, 0, wfP, xfP);
   __builtin_amdgcn_sched_barrier(0);
-
-  for (int kt = 0; kt < nk; ++kt) {
 #ifdef MOE_TRACE
-    if ((blockIdx.x == 8 || blockIdx.x == 1024) && (threadIdx.x & 63) == 0 && kt < 64)
-      moe_dbg[8 * 4096 + (blockIdx.x == 8 ? 0 : 256) + (threadIdx.x >> 6) * 64 + kt] = __builtin_amdgcn_s_memrealtime();
+  unsigned long long tr_v = 0, tr_b = 0, tr_i = 0;
+  const unsigned long long tr0 = __builtin_readcyclecounter();
 #endif
-    read_frags(sa, sw, 1, wfQ, xfQ);
-    __builtin_amdgcn_sched_barrier(0);
-    mma_all(wfP, xfP);
-    __builtin_amdgcn_sched_barrier(0);
-    read_frags(sa, sw, 2, wfP, xfP);
-    __builtin_amdgcn_sched_barrier(0);
-    mma_all(wfQ, xfQ);
-    __builtin_amdgcn_sched_barrier(0);
-    read_frags(sa, sw, 3, wfQ, xfQ);
-    __builtin_amdgcn_sched_barrier(0);
-    mma_all(wfP, xfP);
-    __builtin_amdgcn_sched_barrier(0);
+  for (int kt = 0; kt < nk; ++kt) {
+    // requests of this K tile: W(kt+1) second half, then A(kt+2); W(kt+1)'s
+    // first half went out behind the last MFMA step of tile kt-1
+    const bool do_w = kt >= 1 && kt + 1 < nk, do_a = kt >= 1 && kt + 2 < nk;
+    step(wfP, xfP, wfQ, xfQ, true, sa, sw, 1, [&](int i) { if (do_w) dma_w(kt + 1, fa, 4 + i); });
+    step(wfQ, xfQ, wfP, xfP, true, sa, sw, 2, [&](int i) { if (do_a) dma_a(kt + 2, fw, i); });
+    step(wfP, xfP, wfQ, xfQ, true, sa, sw, 3, [&](int i) { if (do_a) dma_a(kt + 2, fw, 4 + i); });
+    bool next_w = false;
     if (kt + 1 < nk) {
-      // tile kt+1 must have landed (only A(kt+2) may still be outstanding) and
-      // nobody reads the slots of tile kt any more (its last fragment reads
-      // have returned: lgkmcnt(0))
+      // tile kt+1 must have landed (only A(kt+2), the youngest request, may
+      // still be outstanding) and nobody reads the slots of tile kt any more
+      // (its last fragment reads have returned: lgkmcnt(0))
+#ifdef MOE_TRACE
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      const unsigned long long tr1 = __builtin_readcyclecounter();
+#endif
       if (kt + 2 < nk) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
       else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+#ifdef MOE_TRACE
+      const unsigned long long tr2 = __builtin_readcyclecounter();
+#endif
       bare_barrier();
-      if (kt + 2 < nk) issue_w(kt + 2, sa);
-      if (kt + 3 < nk) issue_a(kt + 3, sw);
+#ifdef MOE_TRACE
+      const unsigned long long tr3 = __builtin_readcyclecounter();
+      tr_v += tr2 - tr1; tr_b += tr3 - tr2;
+#endif
+      fa = sa;
+      fw = sw;
       sa = next_slot(sa);
       sw = next_slot(sw);
-      read_frags(sa, sw, 0, wfP, xfP);
+      next_w = kt + 2 < nk;
     }
     __builtin_amdgcn_sched_barrier(0);
-    mma_all(wfQ, xfQ);
-    __builtin_amdgcn_sched_barrier(0);
+    step(wfQ, xfQ, wfP, xfP, kt + 1 < nk, sa, sw, 0, [&](int i) { if (next_w) dma_w(kt + 2, fa, i); });
   }
   wait_vmcnt<0>();
+#ifdef MOE_TRACE
+  if (threadIdx.x == 0 && blockIdx.x < 4096) {
+    unsigned long long* d = moe_dbg + 8 * 4096 + 4 * 128 + blockIdx.x * 4;
+    d[0] = tr_v; d[1] = tr_b; d[2] = tr_i + 0; d[3] = __builtin_readcyclecounter() - tr0;
+  }
+#endif
 }
 
 // Epilogue phase 1: round this wavefront's accumulators to the activation dtype
@@ -691,28 +750,32 @@ template <typename Mma, bool GATED>
 __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams p) {
   using El = typename Mma::El;
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  const int per_xcd = gridDim.x / kXcds;
-  const int logical = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
-  if (logical >= p.num_m_blocks * p.num_n_tiles) return;
+  // only the m-blocks below the padded total are live: cut the per-XCD ranges from
+  // those, so that no XCD is left holding the grid's empty tail
+  const int npp = *p.num_post_pad;
+  const int live_mb = (npp + kBigBM - 1) / kBigBM;
+  const int live = live_mb * p.num_n_tiles;
+  const int per_xcd = (live + kXcds - 1) / kXcds;
+  const int xslot = blockIdx.x / kXcds;
+  const int logical = (blockIdx.x % kXcds) * per_xcd + xslot;
+  if (xslot >= per_xcd || logical >= live) return;
   int nt, mb;
   if (p.m_major) {
     mb = logical / p.num_n_tiles;
     nt = logical - mb * p.num_n_tiles;
   } else {
-    nt = logical / p.num_m_blocks;
-    mb = logical - nt * p.num_m_blocks;
+    nt = logical / live_mb;
+    mb = logical - nt * live_mb;
   }
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lhi = lane >> 5;
   const int wm = wave & 1, wn = wave >> 1;
   [[maybe_unused]] const unsigned long long t_start = MOE_TRACE_NOW();
   [[maybe_unused]] const unsigned long long c_start = __builtin_readcyclecounter();
-  // the three loads below do not depend on each other: one memory latency, not three
-  const int npp = *p.num_post_pad;
+  // the two loads below do not depend on each other: one memory latency, not two
   const int e = p.expert_ids[(mb * kBigBM) / p.align_bs];
   const int64_t my_slot = static_cast<int64_t>(mb) * kBigBM + tid;
   const int my_tok = p.sorted_ids[my_slot < p.sorted_cap ? my_slot : p.sorted_cap - 1];
-  if (mb * kBigBM >= npp) return;
   const int n0 = nt * (GATED ? kBigBNW / 2 : kBigBNW);
   int* s_tok = reinterpret_cast<int*>(smem + kBigLdsBytes);
   float* s_rw_all = reinterpret_cast<float*>(smem + kBigLdsBytes + kBigBM * 4);
@@ -723,7 +786,7 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   if (lane == 0) s_cnt[wave] = wave_cnt;
   __syncthreads();
   const int nvalid = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
-  if (nvalid == 0) return;
+  if (nvalid <= p.cold_max) return;  // empty, or left to the small-block kernel of a split launch
   float my_rw = 1.f;
   if (p.mul_weight) my_rw = my_tok < p.numel ? p.topk_w[my_tok] : 0.f;
 
@@ -850,11 +913,35 @@ int launch(const GemmParams& p, hipStream_t s) {
 // Picks the largest M tile that divides the caller's alignment block size: a
 // block of the aligned list is then a whole number of kernel tiles, all of one
 // expert.
+// Picks the largest M tile that divides the caller's alignment block size: a
+// block of the aligned list is then a whole number of kernel tiles, all of one
+// expert.  With 256-slot blocks the work can be split (kSplitCold): blocks with
+// at most kColdMax real slots (cold experts, and the thin tail block of hot
+// ones) go to the 64-slot kernel, everything else to the large-tile kernel.
+constexpr int kColdMax = 64;
+// Measured at the 8192+256 batch: the split costs more (the cold launch runs alone,
+// latency-bound) than the large-tile kernel gains, so it is off.
+constexpr bool kSplitCold = false;
+
 template <typename Mma, bool GATED>
 int launch_bm(GemmParams& p, int block_size, int64_t sorted_cap, hipStream_t s) {
   p.align_bs = block_size;
+  p.cold_max = -1;
+  p.m_major = 0;
   if constexpr (Mma::kEs == 2) {
-    if (block_size % 256 == 0 && p.Kd % kBigBK == 0) return launch_big<Mma, GATED>(p, sorted_cap, s);
+    if (block_size % 256 == 0 && p.Kd % kBigBK == 0) {
+      if (kSplitCold) {
+        p.cold_max = kColdMax;
+        p.num_m_blocks = static_cast<int>((sorted_cap + 63) / 64);
+        p.num_n_tiles = (p.N + (GATED ? 128 : 256) - 1) / (GATED ? 128 : 256);
+        int rc = launch<Mma, 64, 256, 1, GATED>(p, s);
+        if (rc) return rc;
+      } else {
+        p.cold_max = 0;
+      }
+      p.m_major = 1;  // a token block is reused by all its n-tiles through one L2
+      return launch_big<Mma, GATED>(p, sorted_cap, s);
+    }
   }
   if (block_size % 128 == 0) {
     p.num_m_blocks = static_cast<int>((sorted_cap + 127) / 128);
@@ -966,10 +1053,6 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.limit = a->swiglu_limit;
   p.activation = a->activation;
   p.interleaved = a->activation == MOE_ACT_SWIGLUOAI;
-  // the large-tile kernel reuses a token block across its n-tiles in one L2;
-  // the small-block kernels stream weights and keep a weight strip in one L2
-  p.m_major = (a->block_size % 256 == 0 && a->H % kBigBK == 0 && a->I % kBigBK == 0) ? 1 : 0;
-
   // pass 1: x . W13^T with the gated activation, rows addressed by slot
   p.a = a->x; p.lda = a->H; p.w = a->w13; p.w_stride_e = a->w13_stride_e; p.w_stride_n = a->w13_stride_n;
   p.bias = a->w13_bias; p.bias_stride_e = 2LL * a->I;
