@@ -107,8 +107,6 @@ struct GemmParams {
   float alpha, limit;
   int64_t sorted_cap; // capacity of sorted_ids
   int align_bs;      // block size the alignment was made with (a multiple of the kernel's M tile)
-  int cold_max;      // large-tile kernel: skip alignment blocks with at most this many real slots;
-                     // small-block kernel: when >= 0, take only those blocks (-1: take all)
   int m_major;       // workgroup order inside an XCD: all n-tiles of an m-block are neighbours
 };
 
@@ -124,15 +122,15 @@ __device__ __forceinline__ int swizzled(int row, int chunk) {
 
 // Writes one 32x32 accumulator fragment (pair, when gated): this lane holds, for
 // token `tok` (slot `slot`), the output columns ncol0 + 8*g + i, g,i in 0..3.
+// `rw` is the routed weight of the slot when the pass applies it, else 1.
 // Rounding follows the reference's storage points: the GEMM result is rounded to
 // the activation dtype, silu is rounded, the product is rounded
 // (nanovllm/layers/for_moe/fused_moe.py:216, csrc/activation_kernels.cu:11,23).
 template <typename El, bool GATED>
 __device__ __forceinline__ void store_fragment(const GemmParams& p, int e, const f32x16& ga,
-                                               const f32x16& ua, int tok, int slot, int ncol0) {
+                                               const f32x16& ua, int tok, int slot, int ncol0, float rw) {
   using S = typename El::S;
   const S* bias = static_cast<const S*>(p.bias);
-  const float rw = p.mul_weight ? p.topk_w[tok] : 1.f;
   // fp8: the accumulator is in units of (activation scale x weight scale)
   const float as = p.a_scale ? p.a_scale[p.a_by_slot ? slot : tok / p.top_k] : 1.f;
   const float* ws = p.w_scale ? p.w_scale + e * p.w_scale_stride_e : nullptr;
@@ -229,11 +227,6 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
   }
   // real slots come first in an alignment block: a tile that starts on padding is empty
   if (p.sorted_ids[mb * BM] >= p.numel) return;
-  if (p.cold_max >= 0) {
-    // split launch: this kernel only serves alignment blocks with few real slots
-    const int blk0 = (mb * BM) / p.align_bs * p.align_bs;
-    if (p.cold_max < p.align_bs && p.sorted_ids[blk0 + p.cold_max] < p.numel) return;
-  }
   const int e = p.expert_ids[(mb * BM) / p.align_bs];
   const int n0 = nt * BN_OUT;
 
@@ -348,10 +341,11 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     const int slot = mb * BM + wm * TM + fm * 32 + l32;
     const int tok = p.sorted_ids[slot];
     if (tok >= p.numel) continue;  // padding slot
+    const float rw = p.mul_weight ? p.topk_w[tok] : 1.f;
 #pragma unroll
     for (int fo = 0; fo < FNO; ++fo) {
       const int ncol0 = n0 + (GATED ? wn * (TNW / 2) : wn * TNW) + fo * 32 + 4 * lhi;
-      store_fragment<El, GATED>(p, e, acc[fo][fm], acc[GATED ? fo + FNO : fo][fm], tok, slot, ncol0);
+      store_fragment<El, GATED>(p, e, acc[fo][fm], acc[GATED ? fo + FNO : fo][fm], tok, slot, ncol0, rw);
     }
   }
 }
@@ -786,7 +780,7 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   if (lane == 0) s_cnt[wave] = wave_cnt;
   __syncthreads();
   const int nvalid = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
-  if (nvalid <= p.cold_max) return;  // empty, or left to the small-block kernel of a split launch
+  if (nvalid == 0) return;
   float my_rw = 1.f;
   if (p.mul_weight) my_rw = my_tok < p.numel ? p.topk_w[my_tok] : 0.f;
 
@@ -870,6 +864,200 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
 #endif
 }
 
+
+// ---------------------------------------------------------------------------
+// Streaming variant for bandwidth-bound calls (a few tokens per expert: decode).
+// The time of such a call is the time to pull every active expert's weights
+// out of HBM once, so the kernel is built around that stream: a workgroup owns
+// 64 weight rows of one expert and one alignment block of 32 slots, and walks
+// K in units of 64 elements.  A unit (64 weight rows and 32 token rows of
+// 128 B: 8 KB + 4 KB) goes global->LDS by DMA into a ring of four units, three
+// of them in flight while the fourth is multiplied; three workgroups fit a CU,
+// which keeps about 100 KB per CU on its way from HBM and hides a workgroup's
+// start-up and epilogue behind its neighbours' streams.  Small tiles (256 KB of
+// weights in the gate-up pass) also keep the last wave of workgroups short.
+// All four wavefronts issue DMA requests; the MFMA work of a 32-slot block is
+// so small (8 MFMAs per unit) that wavefront 0 does all of it.  Rows are laid
+// out in LDS like the large-tile kernel's (16-byte chunk c of row r at chunk
+// c ^ ((r >> 1) & 7)).  Everything the start-up reads is wavefront-uniform and
+// comes through the scalar cache, in two round trips.
+// ---------------------------------------------------------------------------
+constexpr int kStBK = 64, kStRowBytes = kStBK * 2, kStRows = 64, kStUnits = 4, kStBM = 32;
+constexpr int kStWBytes = kStRows * kStRowBytes;               // 8 KB of weights per unit
+constexpr int kStUnitBytes = kStWBytes + kStBM * kStRowBytes;  // plus 4 KB of tokens
+constexpr int kStDmaPerUnit = 3;                               // requests per wavefront and unit
+
+template <typename Mma, bool GATED>
+__global__ __launch_bounds__(kThreads, 3) void stream_gemm_kernel(const GemmParams p) {
+  using El = typename Mma::El;
+  __shared__ __attribute__((aligned(1024))) char smem[kStUnits * kStUnitBytes];
+  constexpr int BN_OUT = GATED ? kStRows / 2 : kStRows;
+  // Per-XCD ranges of the (block major, n-tile minor) order, cut from the live
+  // blocks only: the n-tiles of a block run side by side and share its token
+  // rows through one L2 (in the down pass those rows are 1.5 KB x 32 per block
+  // and were re-fetched for every n-tile otherwise).
+  const int live_mb = (*p.num_post_pad + kStBM - 1) / kStBM;
+  const int live = live_mb * p.num_n_tiles;
+  const int per_xcd = (live + kXcds - 1) / kXcds;
+  const int xslot = blockIdx.x / kXcds;
+  const int logical = (blockIdx.x % kXcds) * per_xcd + xslot;
+  if (xslot >= per_xcd || logical >= live) return;
+  int mb = logical / p.num_n_tiles;
+  int nt = logical - mb * p.num_n_tiles;
+  {
+    // Blocks of one expert (it has more than 32 tokens) stream the same weights.
+    // Inside an aligned group of four blocks, reorder a run of g same-expert
+    // blocks from (block, n-tile) to (n-tile, block): the g workgroups that
+    // read one weight tile then start back to back on one XCD and the second
+    // to g-th find the lines in L2 (or already requested).
+    const int q0 = mb & ~3;
+    int eq[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) eq[i] = q0 + i < live_mb ? p.expert_ids[q0 + i] : -1 - i;
+    const int me = mb - q0;
+    int lo = me, hi = me;
+#pragma unroll
+    for (int i = 1; i < 4; ++i) {
+      if (lo == me - i + 1 && lo > 0 && eq[lo - 1] == eq[me]) lo = me - i;
+      if (hi == me + i - 1 && hi < 3 && eq[hi + 1] == eq[me]) hi = me + i;
+    }
+    const int g = hi - lo + 1;
+    const int li = (me - lo) * p.num_n_tiles + nt;
+    nt = li / g;
+    mb = q0 + lo + (li - nt * g);
+  }
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  [[maybe_unused]] const unsigned long long t_start = MOE_TRACE_NOW();
+  const int l32 = lane & 31, lhi = lane >> 5;
+  const int n0 = nt * BN_OUT;
+
+  // second round trip: the expert, and the eight slots whose token rows this wavefront requests
+  const int32_t* sid = p.sorted_ids + static_cast<int64_t>(mb) * kStBM;
+  const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
+  const int first = sid[0];
+  const int4 s0 = *reinterpret_cast<const int4*>(sid + 8 * wave);
+  const int4 s1 = *reinterpret_cast<const int4*>(sid + 8 * wave + 4);
+  if (first >= p.numel) return;  // real slots come first: the block is empty
+  // What the epilogue needs per slot is fetched now, ahead of the stream: a load
+  // issued behind ~100 KB of queued DMA requests would take microseconds to return.
+  int tok = p.numel;
+  float rw = 1.f;
+  if (wave == 0) {
+    tok = sid[l32];
+    if (p.mul_weight && tok < p.numel) rw = p.topk_w[tok];
+  }
+
+  // DMA requests of this wavefront: token rows 8 * wave + lane / 8, weight rows
+  // 16 * wave + 8 * j + lane / 8 (j < 2); lane % 8 is the chunk the lane's 16 bytes land in
+  const char* a_base = static_cast<const char*>(p.a);
+  const char* w_base = static_cast<const char*>(p.w) + static_cast<int64_t>(e) * p.w_stride_e * 2;
+  uint32_t a_off, w_off[2];
+  {
+    const int q = lane >> 3;
+    const int rr = 8 * wave + q;
+    int64_t src = mb * kStBM + rr;
+    if (!p.a_by_slot) {
+      const int lo = (q & 2) ? ((q & 1) ? s0.w : s0.z) : ((q & 1) ? s0.y : s0.x);
+      const int hi = (q & 2) ? ((q & 1) ? s1.w : s1.z) : ((q & 1) ? s1.y : s1.x);
+      const int tok = (q & 4) ? hi : lo;
+      src = tok < p.numel ? tok / p.top_k : 0;
+    }
+    a_off = static_cast<uint32_t>(src * p.lda * 2 + (((lane & 7) ^ ((rr >> 1) & 7)) << 4));
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int rr = 16 * wave + 8 * j + (lane >> 3);
+    int64_t wrow;
+    if constexpr (GATED) {
+      const int half = rr >> 5;
+      int n = n0 + (rr & 31);
+      n = n < p.N ? n : p.N - 1;
+      wrow = p.interleaved ? (2 * n + half) : (half * p.N + n);
+    } else {
+      const int n = n0 + rr;
+      wrow = n < p.N ? n : p.N - 1;
+    }
+    w_off[j] = static_cast<uint32_t>(wrow * p.w_stride_n * 2 + (((lane & 7) ^ ((rr >> 1) & 7)) << 4));
+  }
+  const uint32_t lds0 = lds_offset_of(smem);
+  const uint32_t dma_w = __builtin_amdgcn_readfirstlane(lds0 + 16 * wave * kStRowBytes);
+  const uint32_t dma_a = __builtin_amdgcn_readfirstlane(lds0 + kStWBytes + 8 * wave * kStRowBytes);
+  auto issue = [&](int u) {
+    const uint32_t ring = (u % kStUnits) * kStUnitBytes;
+    lds_dma16(a_base + u * kStRowBytes, a_off, dma_a + ring);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) lds_dma16(w_base + u * kStRowBytes, w_off[j], dma_w + ring + j * 1024);
+  };
+
+  f32x16 acc0, acc1;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
+  const int nu = p.Kd / kStBK;
+  int rd_k[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) rd_k[kk] = l32 * kStRowBytes + (((2 * kk + lhi) ^ ((l32 >> 1) & 7)) << 4);
+
+  [[maybe_unused]] const unsigned long long t_pro = MOE_TRACE_NOW();
+  [[maybe_unused]] unsigned long long t_first = 0;
+  issue(0);
+  if (1 < nu) issue(1);
+  if (2 < nu) issue(2);
+  for (int u = 0; u < nu; ++u) {
+    // unit u has landed (only the two younger units may be outstanding) and
+    // wavefront 0 is done reading unit u-1, whose ring slot the next request reuses
+    if (u + 2 < nu) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * kStDmaPerUnit) : "memory");
+    else if (u + 1 < nu) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kStDmaPerUnit) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    bare_barrier();
+#ifdef MOE_TRACE
+    if (u == 0) t_first = MOE_TRACE_NOW();
+#endif
+    if (u + 3 < nu) issue(u + 3);
+    if (wave == 0) {
+      const char* st = smem + (u % kStUnits) * kStUnitBytes;
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const uint4 x = *reinterpret_cast<const uint4*>(st + kStWBytes + rd_k[kk]);
+        const uint4 w0 = *reinterpret_cast<const uint4*>(st + rd_k[kk]);
+        const uint4 w1 = *reinterpret_cast<const uint4*>(st + 32 * kStRowBytes + rd_k[kk]);
+        acc0 = Mma::mma(w0, x, acc0);
+        acc1 = Mma::mma(w1, x, acc1);
+      }
+    }
+  }
+
+  if (wave != 0) return;
+  [[maybe_unused]] const unsigned long long t_loop = MOE_TRACE_NOW();
+  const int slot = mb * kStBM + l32;
+  if (tok < p.numel) {
+    if constexpr (GATED) {
+      store_fragment<El, true>(p, e, acc0, acc1, tok, slot, n0 + 4 * lhi, rw);
+    } else {
+      store_fragment<El, false>(p, e, acc0, acc0, tok, slot, n0 + 4 * lhi, rw);
+      store_fragment<El, false>(p, e, acc1, acc1, tok, slot, n0 + 32 + 4 * lhi, rw);
+    }
+  }
+#ifdef MOE_TRACE
+  if (tid == 0 && blockIdx.x < 4096) {
+    moe_dbg[blockIdx.x * 8 + 0] = t_start; moe_dbg[blockIdx.x * 8 + 1] = t_pro;
+    moe_dbg[blockIdx.x * 8 + 2] = t_first; moe_dbg[blockIdx.x * 8 + 3] = t_loop;
+    moe_dbg[blockIdx.x * 8 + 4] = MOE_TRACE_NOW(); moe_dbg[blockIdx.x * 8 + 5] = __builtin_amdgcn_s_getreg((20) | (0 << 6) | (3 << 11));
+  }
+#endif
+}
+
+template <typename Mma, bool GATED>
+int launch_stream(GemmParams& p, int64_t sorted_cap, hipStream_t s) {
+  p.num_m_blocks = static_cast<int>((sorted_cap + kStBM - 1) / kStBM);
+  p.num_n_tiles = (p.N + (GATED ? kStRows / 2 : kStRows) - 1) / (GATED ? kStRows / 2 : kStRows);
+  const int64_t tiles = static_cast<int64_t>(p.num_m_blocks) * p.num_n_tiles;
+  const int64_t grid = (tiles + kXcds - 1) / kXcds * kXcds;
+  if (grid > INT32_MAX) return moe_fail(MOE_ERR_ARG, "fused_experts: grid of %lld workgroups", static_cast<long long>(grid));
+  hipLaunchKernelGGL((stream_gemm_kernel<Mma, GATED>), dim3(static_cast<unsigned>(grid)), dim3(kThreads), 0, s, p);
+  return moe_check_launch(GATED ? "fused_experts (gate-up pass)" : "fused_experts (down pass)");
+}
+
 template <typename Mma, bool GATED>
 int launch_big(GemmParams& p, int64_t sorted_cap, hipStream_t s) {
   constexpr int lds = kBigLdsTotal;
@@ -910,38 +1098,25 @@ int launch(const GemmParams& p, hipStream_t s) {
   return moe_check_launch(GATED ? "fused_experts (gate-up pass)" : "fused_experts (down pass)");
 }
 
-// Picks the largest M tile that divides the caller's alignment block size: a
-// block of the aligned list is then a whole number of kernel tiles, all of one
+// Picks the kernel by the caller's alignment block size.  16-bit dtypes: blocks
+// of 256 slots go to the large-tile kernel (compute-bound calls), blocks of 32
+// slots to the streaming kernel (bandwidth-bound calls).  Everything
+// else runs on the register-staged kernels with the largest M tile that
+// divides the block size, so that a block is a whole number of tiles of one
 // expert.
-// Picks the largest M tile that divides the caller's alignment block size: a
-// block of the aligned list is then a whole number of kernel tiles, all of one
-// expert.  With 256-slot blocks the work can be split (kSplitCold): blocks with
-// at most kColdMax real slots (cold experts, and the thin tail block of hot
-// ones) go to the 64-slot kernel, everything else to the large-tile kernel.
-constexpr int kColdMax = 64;
-// Measured at the 8192+256 batch: the split costs more (the cold launch runs alone,
-// latency-bound) than the large-tile kernel gains, so it is off.
-constexpr bool kSplitCold = false;
-
 template <typename Mma, bool GATED>
 int launch_bm(GemmParams& p, int block_size, int64_t sorted_cap, hipStream_t s) {
   p.align_bs = block_size;
-  p.cold_max = -1;
   p.m_major = 0;
   if constexpr (Mma::kEs == 2) {
     if (block_size % 256 == 0 && p.Kd % kBigBK == 0) {
-      if (kSplitCold) {
-        p.cold_max = kColdMax;
-        p.num_m_blocks = static_cast<int>((sorted_cap + 63) / 64);
-        p.num_n_tiles = (p.N + (GATED ? 128 : 256) - 1) / (GATED ? 128 : 256);
-        int rc = launch<Mma, 64, 256, 1, GATED>(p, s);
-        if (rc) return rc;
-      } else {
-        p.cold_max = 0;
-      }
       p.m_major = 1;  // a token block is reused by all its n-tiles through one L2
       return launch_big<Mma, GATED>(p, sorted_cap, s);
     }
+    // byte offsets of token rows are 32-bit in the streaming kernel
+    const int64_t a_rows = p.a_by_slot ? sorted_cap : p.numel / p.top_k;
+    if (block_size == kStBM && p.Kd % kStBK == 0 && a_rows * p.lda * 2 < (1LL << 32))
+      return launch_stream<Mma, GATED>(p, sorted_cap, s);
   }
   if (block_size % 128 == 0) {
     p.num_m_blocks = static_cast<int>((sorted_cap + 127) / 128);
