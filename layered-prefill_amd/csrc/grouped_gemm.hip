@@ -865,6 +865,47 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
 }
 
 
+// Epilogue of the streaming kernel for full, aligned 16-bit tiles: same storage
+// points as store_fragment, with the hardware conversions and the fast SiLU of
+// the large-tile epilogue (one wavefront finishes the whole tile, so the
+// instruction count is the epilogue's latency).
+template <typename El, bool GATED, int ACT>
+__device__ __forceinline__ void stream_store(const GemmParams& p, int e, const f32x16& ga, const f32x16& ua,
+                                             int tok, int slot, int ncol0, float rw) {
+  using S = typename El::S;
+  const S* bias = static_cast<const S*>(p.bias);
+  const int64_t crow = p.a_by_slot ? tok : slot;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int n = ncol0 + 8 * g;
+    float gv[4], uv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      gv[i] = ga[4 * g + i];
+      uv[i] = ua[4 * g + i];
+      if (bias) {
+        if constexpr (GATED) {
+          gv[i] += El::ld(bias[e * p.bias_stride_e + (p.interleaved ? 2 * (n + i) : n + i)]);
+          uv[i] += El::ld(bias[e * p.bias_stride_e + (p.interleaved ? 2 * (n + i) + 1 : p.N + n + i)]);
+        } else {
+          gv[i] += El::ld(bias[e * p.bias_stride_e + n + i]);
+        }
+      }
+      gv[i] *= rw;
+      uv[i] *= rw;
+    }
+    uint2 out;
+    if constexpr (GATED) {
+      out.x = gated_pair<El, ACT>(p, pack2<El>(gv[0], gv[1]), pack2<El>(uv[0], uv[1]));
+      out.y = gated_pair<El, ACT>(p, pack2<El>(gv[2], gv[3]), pack2<El>(uv[2], uv[3]));
+    } else {
+      out.x = pack2<El>(gv[0], gv[1]);
+      out.y = pack2<El>(gv[2], gv[3]);
+    }
+    *reinterpret_cast<uint2*>(static_cast<S*>(p.c) + crow * p.ldc + n) = out;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Streaming variant for bandwidth-bound calls (a few tokens per expert: decode).
 // The time of such a call is the time to pull every active expert's weights
@@ -1031,8 +1072,15 @@ __global__ __launch_bounds__(kThreads, 3) void stream_gemm_kernel(const GemmPara
   [[maybe_unused]] const unsigned long long t_loop = MOE_TRACE_NOW();
   const int slot = mb * kStBM + l32;
   if (tok < p.numel) {
+    const bool fast = n0 + BN_OUT <= p.N && (p.ldc & 3) == 0 && !p.w_scale;
     if constexpr (GATED) {
-      store_fragment<El, true>(p, e, acc0, acc1, tok, slot, n0 + 4 * lhi, rw);
+      if (!fast) store_fragment<El, true>(p, e, acc0, acc1, tok, slot, n0 + 4 * lhi, rw);
+      else if (p.activation == MOE_ACT_SILU) stream_store<El, true, MOE_ACT_SILU>(p, e, acc0, acc1, tok, slot, n0 + 4 * lhi, rw);
+      else if (p.activation == MOE_ACT_SWIGLUOAI) stream_store<El, true, MOE_ACT_SWIGLUOAI>(p, e, acc0, acc1, tok, slot, n0 + 4 * lhi, rw);
+      else stream_store<El, true, MOE_ACT_GELU>(p, e, acc0, acc1, tok, slot, n0 + 4 * lhi, rw);
+    } else if (fast) {
+      stream_store<El, false, 0>(p, e, acc0, acc0, tok, slot, n0 + 4 * lhi, rw);
+      stream_store<El, false, 0>(p, e, acc1, acc1, tok, slot, n0 + 32 + 4 * lhi, rw);
     } else {
       store_fragment<El, false>(p, e, acc0, acc0, tok, slot, n0 + 4 * lhi, rw);
       store_fragment<El, false>(p, e, acc1, acc1, tok, slot, n0 + 32 + 4 * lhi, rw);
