@@ -98,6 +98,33 @@ def time_steps(layer: Layer, steps: int, warmup: int):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
+def time_graph_replays(layer: Layer, steps: int, warmup: int):
+    """The same step recorded once into a HIP graph and replayed: what a serving
+    loop that captures its decode iteration pays (the reference runs this layer
+    inside captured graph segments, nanovllm/models/qwen3_moe.py:673-759).
+    Returns (ms per replay, max |graph - eager| of the output)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            layer.step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    eager = layer.step().float()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = layer.step()
+    for _ in range(warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    return ms, float((out.float() - eager).abs().max())
+
+
 def time_stages(layer: Layer, steps: int):
     names = ["topk_softmax", "moe_align_block_size", "gate_up_gemm_act", "down_gemm_weighted",
              "topk_combine"]
@@ -199,6 +226,7 @@ def main() -> int:
                     help="config 4 (chunk amplification) leg: both sides, one side only (for "
                          "rocprofv3 counter runs), or off")
     ap.add_argument("--no-fp8", action="store_true", help="skip the e4m3 leg (config 5)")
+    ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay of the decode leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device copies, the known-size kernel that "
                          "FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -315,6 +343,12 @@ def main() -> int:
                          "hbm_gbs": round(dgbs, 1), "frac_of_hbm_peak": round(dgbs / PEAK_HBM_GBS, 4),
                          "active_experts": dact, "block_size_m": dec.bm,
                          "stage_ms": {k: round(v, 4) for k, v in dstages.items()}}
+        if not a.no_graph:
+            gms, gerr = time_graph_replays(dec, max(a.steps, 50), max(a.warmup, 10))
+            ggbs = dbytes / (gms * 1e-3) / 1e9
+            out["decode"]["hip_graph"] = {"ms_per_step": round(gms, 4), "hbm_gbs": round(ggbs, 1),
+                                          "frac_of_hbm_peak": round(ggbs / PEAK_HBM_GBS, 4),
+                                          "max_abs_diff_vs_eager": gerr}
         del dec
 
     if not a.no_cpu_baseline:

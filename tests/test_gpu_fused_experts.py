@@ -257,3 +257,36 @@ def test_fp8_layered_prefill_batch_sampled_rows(moe, oracle, dev):
     ref = oracle.fused_experts_fp8_ref(x[rows], w13q.view(torch.uint8).cpu(), w13s.cpu(),
                                        w2q.view(torch.uint8).cpu(), w2s.cpu(), tw.cpu()[rows], ids.cpu()[rows])
     _close_fp8(out[rows.to(dev)], ref)
+
+
+def test_layer_step_replays_from_a_hip_graph(moe, oracle, dev):
+    """Routing, alignment and the expert MLP enqueue no allocation of their own,
+    no host sync and no memset, so one call can be recorded into a HIP graph.
+    Every replay, with eager work and synchronisations in between, must give
+    the eager result bit for bit (all kernels are deterministic)."""
+    x, w13, w2, logits = _layer(16, 256, 128, 96, 4, 23, torch.bfloat16)
+    x, w13, w2, logits = x.to(dev), w13.to(dev), w2.to(dev), logits.to(dev)
+
+    def step(inp):
+        tw, ids, _ = moe.fused_topk(inp, logits, 4, True)
+        return moe.fused_experts(inp, w13, w2, None, None, tw, ids)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step(x)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    static_x = x.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = step(static_x)
+    for r in range(4):
+        fresh = (x * (1.0 + 0.25 * r)).to(torch.bfloat16)
+        want = step(fresh).clone()          # eager work between replays
+        torch.cuda.synchronize()
+        static_x.copy_(fresh)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_out, want), f"replay {r} differs from the eager result"
