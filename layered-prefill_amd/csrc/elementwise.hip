@@ -113,6 +113,66 @@ __global__ __launch_bounds__(kThreads) void quant_rows_e4m3_kernel(
   for (int c = lane; c < cols; c += kWave) q[row * cols + c] = f32_to_e4m3(El::ld(src[c]) / s);
 }
 
+// 16-bit sources with up to NV * 512 columns: the row stays in registers between
+// the amax pass and the conversion, 16 bytes in and 8 bytes out per lane and
+// step.  Same arithmetic as the kernel above, element by element.
+template <typename El, int NV>
+__global__ __launch_bounds__(kThreads) void quant_rows_e4m3_vec_kernel(
+    const typename El::S* __restrict__ w, int64_t rows, int cols, uint8_t* __restrict__ q,
+    float* __restrict__ scales) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t row = blockIdx.x * static_cast<int64_t>(kThreads / kWave) + threadIdx.x / kWave;
+  if (row >= rows) return;
+  const uint4* src = reinterpret_cast<const uint4*>(w + row * cols);
+  const int nvec = cols / 8;
+  uint4 v[NV];
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = lane + i * kWave;
+    v[i] = c < nvec ? src[c] : uint4{0, 0, 0, 0};
+    const uint32_t wds[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      amax = fmaxf(amax, fabsf(El::ld(static_cast<uint16_t>(wds[j]))));
+      amax = fmaxf(amax, fabsf(El::ld(static_cast<uint16_t>(wds[j] >> 16))));
+    }
+  }
+#pragma unroll
+  for (int m = 32; m > 0; m /= 2) amax = fmaxf(amax, __shfl_xor(amax, m, kWave));
+  const float s = amax > 0.f ? amax / 448.f : 1.f;
+  if (lane == 0) scales[row] = s;
+  uint2* dst = reinterpret_cast<uint2*>(q + row * cols);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = lane + i * kWave;
+    if (c >= nvec) continue;
+    const uint32_t wds[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+    uint32_t o[2] = {0, 0};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t lo = f32_to_e4m3(El::ld(static_cast<uint16_t>(wds[j])) / s);
+      const uint32_t hi = f32_to_e4m3(El::ld(static_cast<uint16_t>(wds[j] >> 16)) / s);
+      o[j >> 1] |= (lo | (hi << 8)) << (16 * (j & 1));
+    }
+    dst[c] = uint2{o[0], o[1]};
+  }
+}
+
+template <typename El>
+bool launch_quant_vec(const void* w, int64_t rows, int cols, uint8_t* q, float* scales, dim3 grid,
+                      hipStream_t s) {
+  using S = typename El::S;
+  if (cols % 8 != 0 || cols > 4096 || (reinterpret_cast<uintptr_t>(w) & 15u) || (reinterpret_cast<uintptr_t>(q) & 7u))
+    return false;
+  const int nv = (cols / 8 + kWave - 1) / kWave;
+  const S* src = static_cast<const S*>(w);
+  if (nv <= 2) hipLaunchKernelGGL((quant_rows_e4m3_vec_kernel<El, 2>), grid, dim3(kThreads), 0, s, src, rows, cols, q, scales);
+  else if (nv <= 4) hipLaunchKernelGGL((quant_rows_e4m3_vec_kernel<El, 4>), grid, dim3(kThreads), 0, s, src, rows, cols, q, scales);
+  else hipLaunchKernelGGL((quant_rows_e4m3_vec_kernel<El, 8>), grid, dim3(kThreads), 0, s, src, rows, cols, q, scales);
+  return true;
+}
+
 int grid_for(int64_t work_items) {
   int64_t b = (work_items + kThreads - 1) / kThreads;
   const int64_t cap = 256 * 16;  // 256 CUs, 16 workgroups each; the loops stride past this
@@ -222,10 +282,12 @@ MOE_EXPORT int moe_quant_rows_e4m3(const void* w, int src_dtype, int64_t rows, i
       hipLaunchKernelGGL(quant_rows_e4m3_kernel<ElemF32>, grid, block, 0, s, static_cast<const float*>(w), rows, cols, q, scales);
       break;
     case MOE_F16:
-      hipLaunchKernelGGL(quant_rows_e4m3_kernel<ElemF16>, grid, block, 0, s, static_cast<const uint16_t*>(w), rows, cols, q, scales);
+      if (!launch_quant_vec<ElemF16>(w, rows, cols, q, scales, grid, s))
+        hipLaunchKernelGGL(quant_rows_e4m3_kernel<ElemF16>, grid, block, 0, s, static_cast<const uint16_t*>(w), rows, cols, q, scales);
       break;
     case MOE_BF16:
-      hipLaunchKernelGGL(quant_rows_e4m3_kernel<ElemBF16>, grid, block, 0, s, static_cast<const uint16_t*>(w), rows, cols, q, scales);
+      if (!launch_quant_vec<ElemBF16>(w, rows, cols, q, scales, grid, s))
+        hipLaunchKernelGGL(quant_rows_e4m3_kernel<ElemBF16>, grid, block, 0, s, static_cast<const uint16_t*>(w), rows, cols, q, scales);
       break;
     default:
       return moe_fail(MOE_ERR_ARG, "quant_rows_e4m3: unsupported source dtype code %d", src_dtype);

@@ -36,17 +36,25 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 struct MmaBF16 {
   using El = ElemBF16;
   static constexpr int kEs = 2;  // bytes per input element
+  static constexpr int kBigChunks = 1;  // large-tile kernel: 16-byte chunks per lane and MFMA step
   static __device__ __forceinline__ f32x16 mma(const uint4& a, const uint4& b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x16 mma_big(const uint4 (&a)[1], const uint4 (&b)[1], f32x16 c) {
+    return mma(a[0], b[0], c);
   }
 };
 struct MmaF16 {
   using El = ElemF16;
   static constexpr int kEs = 2;
+  static constexpr int kBigChunks = 1;
   static __device__ __forceinline__ f32x16 mma(const uint4& a, const uint4& b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x16 mma_big(const uint4 (&a)[1], const uint4 (&b)[1], f32x16 c) {
+    return mma(a[0], b[0], c);
   }
 };
 
@@ -77,6 +85,25 @@ struct MmaE4M3 {
     const long b1 = static_cast<long>(b.z) | (static_cast<long>(b.w) << 32);
     c = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a0, b0, c, 0, 0, 0);
     return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a1, b1, c, 0, 0, 0);
+  }
+};
+
+// e4m3 in the large-tile kernel: v_mfma_f32_32x32x64_f8f6f4 takes 32 bytes per
+// lane and operand (K = 64 per step, elements 32 * (lane / 32) .. + 31 of the
+// lane's row) and runs at twice the rate of the 16-bit and the older fp8
+// instructions.  The block scales are fixed at 2^0 (E8M0 127).
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+template <typename OutEl>
+struct MmaE4M3Big {
+  using El = OutEl;
+  static constexpr int kEs = 1;
+  static constexpr int kBigChunks = 2;
+  static __device__ __forceinline__ f32x16 mma_big(const uint4 (&a)[2], const uint4 (&b)[2], f32x16 c) {
+    const i32x8 av = {static_cast<int>(a[0].x), static_cast<int>(a[0].y), static_cast<int>(a[0].z), static_cast<int>(a[0].w),
+                      static_cast<int>(a[1].x), static_cast<int>(a[1].y), static_cast<int>(a[1].z), static_cast<int>(a[1].w)};
+    const i32x8 bv = {static_cast<int>(b[0].x), static_cast<int>(b[0].y), static_cast<int>(b[0].z), static_cast<int>(b[0].w),
+                      static_cast<int>(b[1].x), static_cast<int>(b[1].y), static_cast<int>(b[1].z), static_cast<int>(b[1].w)};
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, 0, 0, 0, 127, 0, 127);
   }
 };
 
@@ -383,7 +410,7 @@ constexpr int kBigDmaPerUnit = 8;                  // global_load_lds instructio
 constexpr int kEpiRowBytes = 128 * 2 + 16;   // one token row of a wavefront's tile, padded
 constexpr int kEpiWaveBytes = 128 * kEpiRowBytes;
 constexpr int kBigLdsBytes = 4 * kEpiWaveBytes;    // epilogue staging, reuses the ring
-constexpr int kBigSideBytes = 2 * kBigBM * 4;      // per-slot token id and routed weight for the epilogue
+constexpr int kBigSideBytes = 3 * kBigBM * 4;      // per-slot token id, routed weight and fp8 row scale for the epilogue
 constexpr int kBigLdsTotal = kBigUnits * kBigUnitBytes;  // the whole 160 KB of the CU
 static_assert(kBigLdsBytes + kBigSideBytes + 16 <= kBigLdsTotal, "epilogue staging must fit in the ring");
 
@@ -450,21 +477,26 @@ struct BigCtx {
   int w_row[4];         // byte offsets of this wavefront's weight fragments in a weight unit
 };
 
+template <int V>
+struct IntTag { static constexpr int value = V; };
+
 // Main loop for a wavefront that has FMC live token fragments (0..4).
 // Unit j of the stream  A(0) W(0) A(1) W(1) ...  lives in ring slot j % 5.
-// One K tile is four MFMA steps; two register sets of fragments (P, Q)
-// alternate, and every step carries, between its MFMAs, the LDS reads of the
-// next step's fragments and four of the sixteen DMA requests of the K tile:
-//   step P(kt,0) reads Q(kt,1), requests W(kt+1)[4..7]
-//   step Q(kt,1) reads P(kt,2), requests A(kt+2)[0..3]
-//   step P(kt,2) reads Q(kt,3), requests A(kt+2)[4..7]
+// One K tile (128 bytes per row) is STEPS MFMA steps of CH 16-byte chunks per
+// lane and operand: four steps of one chunk for the 16-bit dtypes, two steps
+// of two chunks for e4m3.  Two register sets of fragments (P, Q) alternate,
+// and every step carries, between its MFMAs, the LDS reads of the next step's
+// fragments and its share of the sixteen DMA requests of the K tile:
+//   steps 0 .. STEPS-2 of tile kt request W(kt+1)[4..7] and A(kt+2)[0..7]
 //   wait for tile kt+1, barrier (frees the two slots of tile kt)
-//   step Q(kt,3) reads P(kt+1,0), requests W(kt+2)[0..3]
+//   step STEPS-1 reads P(kt+1,0) and requests W(kt+2)[0..3]
 // At the wait only A(kt+2), the youngest request, may still be outstanding.
 // sched_barrier pins this order against the compiler's scheduler.
 template <typename Mma, int FMC>
 __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, int nk,
                                              f32x16 (&acc)[4][4]) {
+  constexpr int CH = Mma::kBigChunks, STEPS = 4 / CH;
+  constexpr int PER = 12 / (STEPS - 1);  // requests carried by each of the first STEPS-1 steps
   auto dma_a = [&](int kt, int slot, int i) {
     lds_dma16(c.a_base + kt * kBigRowBytes, c.a_off[i], c.dma_lds + slot * kBigUnitBytes + i * 4096);
   };
@@ -480,33 +512,40 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
     for (int i = 0; i < 8; ++i) dma_w(kt, slot, i);
   };
   constexpr int XF = FMC > 0 ? FMC : 1;
-  auto read_frags = [&](int sa, int sw, int kk, uint4 (&wf)[4], uint4 (&xf)[XF]) {
+  auto read_frags = [&](int sa, int sw, int kk, uint4 (&wf)[4][CH], uint4 (&xf)[XF][CH]) {
     if constexpr (FMC > 0) {
-      const char* stw = smem + sw * kBigUnitBytes + c.rd_k[kk];
-      const char* sta = smem + sa * kBigUnitBytes + c.x_row + c.rd_k[kk];
 #pragma unroll
-      for (int fn = 0; fn < 4; ++fn) wf[fn] = *reinterpret_cast<const uint4*>(stw + c.w_row[fn]);
+      for (int ch = 0; ch < CH; ++ch) {
+        const char* stw = smem + sw * kBigUnitBytes + c.rd_k[kk * CH + ch];
+        const char* sta = smem + sa * kBigUnitBytes + c.x_row + c.rd_k[kk * CH + ch];
 #pragma unroll
-      for (int fm = 0; fm < FMC; ++fm)
-        xf[fm] = *reinterpret_cast<const uint4*>(sta + fm * 32 * kBigRowBytes);
+        for (int fn = 0; fn < 4; ++fn) wf[fn][ch] = *reinterpret_cast<const uint4*>(stw + c.w_row[fn]);
+#pragma unroll
+        for (int fm = 0; fm < FMC; ++fm)
+          xf[fm][ch] = *reinterpret_cast<const uint4*>(sta + fm * 32 * kBigRowBytes);
+      }
     }
   };
   // One MFMA step on fragment set X.  The LDS reads of the next step's set Y
-  // and four DMA requests are spread between its MFMAs instead of being issued
+  // and ND DMA requests are spread between its MFMAs instead of being issued
   // back to back: the LDS and the vector memory path each take one wavefront
   // request every few dozen clocks when all four wavefronts stream, so a burst
   // stalls the wavefront, and with it the matrix pipe, until the queue drains.
   // Reads go out in the order the next step consumes them.
-  auto step = [&](const uint4 (&wfX)[4], const uint4 (&xfX)[XF], uint4 (&wfY)[4], uint4 (&xfY)[XF],
-                  bool load_y, int ya, int yw, int ykk, auto&& dma) {
-    const char* stw = smem + yw * kBigUnitBytes + c.rd_k[ykk];
-    const char* sta = smem + ya * kBigUnitBytes + c.x_row + c.rd_k[ykk];
+  auto step = [&](auto nd_tag, const uint4 (&wfX)[4][CH], const uint4 (&xfX)[XF][CH], uint4 (&wfY)[4][CH],
+                  uint4 (&xfY)[XF][CH], bool load_y, int ya, int yw, int ykk, auto&& dma) {
+    constexpr int ND = decltype(nd_tag)::value;
     auto read_y = [&](int r) {  // r: 0 x0, 1..4 w0..w3, 5.. x1..
       if constexpr (FMC > 0) {
         if (!load_y) return;
-        if (r == 0) xfY[0] = *reinterpret_cast<const uint4*>(sta);
-        else if (r <= 4) wfY[r - 1] = *reinterpret_cast<const uint4*>(stw + c.w_row[r - 1]);
-        else if (r - 4 < FMC) xfY[r - 4] = *reinterpret_cast<const uint4*>(sta + (r - 4) * 32 * kBigRowBytes);
+#pragma unroll
+        for (int ch = 0; ch < CH; ++ch) {
+          const char* stw = smem + yw * kBigUnitBytes + c.rd_k[ykk * CH + ch];
+          const char* sta = smem + ya * kBigUnitBytes + c.x_row + c.rd_k[ykk * CH + ch];
+          if (r == 0) xfY[0][ch] = *reinterpret_cast<const uint4*>(sta);
+          else if (r <= 4) wfY[r - 1][ch] = *reinterpret_cast<const uint4*>(stw + c.w_row[r - 1]);
+          else if (r - 4 < FMC) xfY[r - 4][ch] = *reinterpret_cast<const uint4*>(sta + (r - 4) * 32 * kBigRowBytes);
+        }
       }
     };
     constexpr int NM = 4 * FMC;  // MFMAs of this step
@@ -514,21 +553,24 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
     for (int m = 0; m < (NM > 0 ? NM : 1); ++m) {
       if constexpr (NM > 0) {
         const int fm = m >> 2, fn = m & 3;
-        acc[fn][fm] = Mma::mma(wfX[fn], xfX[fm], acc[fn][fm]);
+        acc[fn][fm] = Mma::mma_big(wfX[fn], xfX[fm], acc[fn][fm]);
       }
       __builtin_amdgcn_sched_barrier(0);
       if ((m & 1) == 0) read_y(m >> 1);
-      if ((m & 3) == 3) dma(m >> 2);
+#pragma unroll
+      for (int j = (m * ND) / 16; j < ((m + 1) * ND) / 16; ++j) dma(j);
       __builtin_amdgcn_sched_barrier(0);
     }
     // wavefronts with fewer live fragments have fewer MFMAs to hide requests behind
 #pragma unroll
     for (int r = (NM + 1) / 2; r < 8; ++r) read_y(r);
 #pragma unroll
-    for (int i = NM / 4; i < 4; ++i) dma(i);
+    for (int j = ((NM > 0 ? NM : 1) * ND) / 16; j < ND; ++j) dma(j);
     __builtin_amdgcn_sched_barrier(0);
   };
   auto next_slot = [](int s) { return s + 2 >= kBigUnits ? s + 2 - kBigUnits : s + 2; };
+  using Tag4 = IntTag<4>;
+  using TagPer = IntTag<PER>;
 
   // fill the ring: A(0) W(0) A(1) W(1) A(2), then wait for tile 0 only
   issue_a(0, 0);
@@ -541,7 +583,7 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
   bare_barrier();
   int sa = 0, sw = 1;  // slots of the tile being multiplied
   int fa = 0, fw = 0;  // slots the previous tile left free: W(kt+1) goes to fa, A(kt+2) to fw
-  uint4 wfP[4], xfP[XF], wfQ[4], xfQ[XF];
+  uint4 wfP[4][CH], xfP[XF][CH], wfQ[4][CH], xfQ[XF][CH];
   read_frags(sa, sw, 0, wfP, xfP);
   __builtin_amdgcn_sched_barrier(0);
 #ifdef MOE_TRACE
@@ -549,12 +591,20 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
   const unsigned long long tr0 = __builtin_readcyclecounter();
 #endif
   for (int kt = 0; kt < nk; ++kt) {
-    // requests of this K tile: W(kt+1) second half, then A(kt+2); W(kt+1)'s
+    // requests of this K tile, in order: W(kt+1) second half, then A(kt+2); W(kt+1)'s
     // first half went out behind the last MFMA step of tile kt-1
     const bool do_w = kt >= 1 && kt + 1 < nk, do_a = kt >= 1 && kt + 2 < nk;
-    step(wfP, xfP, wfQ, xfQ, true, sa, sw, 1, [&](int i) { if (do_w) dma_w(kt + 1, fa, 4 + i); });
-    step(wfQ, xfQ, wfP, xfP, true, sa, sw, 2, [&](int i) { if (do_a) dma_a(kt + 2, fw, i); });
-    step(wfP, xfP, wfQ, xfQ, true, sa, sw, 3, [&](int i) { if (do_a) dma_a(kt + 2, fw, 4 + i); });
+    auto req = [&](int q) {
+      if (q < 4) { if (do_w) dma_w(kt + 1, fa, 4 + q); }
+      else { if (do_a) dma_a(kt + 2, fw, q - 4); }
+    };
+    if constexpr (STEPS == 4) {
+      step(TagPer{}, wfP, xfP, wfQ, xfQ, true, sa, sw, 1, [&](int j) { req(j); });
+      step(TagPer{}, wfQ, xfQ, wfP, xfP, true, sa, sw, 2, [&](int j) { req(PER + j); });
+      step(TagPer{}, wfP, xfP, wfQ, xfQ, true, sa, sw, 3, [&](int j) { req(2 * PER + j); });
+    } else {
+      step(TagPer{}, wfP, xfP, wfQ, xfQ, true, sa, sw, 1, [&](int j) { req(j); });
+    }
     bool next_w = false;
     if (kt + 1 < nk) {
       // tile kt+1 must have landed (only A(kt+2), the youngest request, may
@@ -581,7 +631,7 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
       next_w = kt + 2 < nk;
     }
     __builtin_amdgcn_sched_barrier(0);
-    step(wfQ, xfQ, wfP, xfP, kt + 1 < nk, sa, sw, 0, [&](int i) { if (next_w) dma_w(kt + 2, fa, i); });
+    step(Tag4{}, wfQ, xfQ, wfP, xfP, kt + 1 < nk, sa, sw, 0, [&](int i) { if (next_w) dma_w(kt + 2, fa, i); });
   }
   wait_vmcnt<0>();
 #ifdef MOE_TRACE
@@ -595,14 +645,37 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
 // Epilogue phase 1: round this wavefront's accumulators to the activation dtype
 // (after the optional bias and routed weight) and park them in its LDS window
 // as [token row][weight row].
-template <typename El, int FMC, bool GATED>
+template <typename El, int FMC, bool GATED, bool SCALED>
 __device__ __forceinline__ void big_park(const GemmParams& p, int e, int n0, int wn, int lhi, int l32,
-                                         const float* s_rw, char* epi, const f32x16 (&acc)[4][4]) {
+                                         const float* s_rw, const float* s_as, char* epi,
+                                         const f32x16 (&acc)[4][4]) {
   using S = typename El::S;
   const S* bias = static_cast<const S*>(p.bias);
+  // weight row (output channel) behind accumulator element (fn, 4 * g + i) of this lane
+  auto wrow_of = [&](int fn, int g, int i) -> int64_t {
+    const int local = fn * 32 + 8 * g + 4 * lhi + i;  // column inside the wavefront tile
+    if constexpr (GATED) {
+      int col = n0 + wn * 64 + (local & 63);
+      col = col < p.N ? col : p.N - 1;
+      const int half = local >> 6;
+      return p.interleaved ? 2 * col + half : half * p.N + col;
+    } else {
+      const int col = n0 + wn * 128 + local;
+      return col < p.N ? col : p.N - 1;
+    }
+  };
+  // e4m3: the accumulator is in units of (row scale of the A operand) x (weight row scale)
+  float ws[SCALED ? 64 : 1];
+  if constexpr (SCALED) {
+#pragma unroll
+    for (int fn = 0; fn < 4; ++fn)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) ws[fn * 16 + q] = p.w_scale[e * p.w_scale_stride_e + wrow_of(fn, q >> 2, q & 3)];
+  }
 #pragma unroll
   for (int fm = 0; fm < FMC; ++fm) {
     const float rw = s_rw[fm * 32 + l32];  // 1 when the routed weight is not applied here
+    [[maybe_unused]] const float as = SCALED ? s_as[fm * 32 + l32] : 1.f;
     char* row = epi + (fm * 32 + l32) * kEpiRowBytes;
 #pragma unroll
     for (int fn = 0; fn < 4; ++fn) {
@@ -611,22 +684,13 @@ __device__ __forceinline__ void big_park(const GemmParams& p, int e, int n0, int
         float v[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] = acc[fn][fm][4 * g + i];
+        if constexpr (SCALED) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] *= as * ws[fn * 16 + 4 * g + i];
+        }
         if (bias) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int local = fn * 32 + 8 * g + 4 * lhi + i;  // column inside the wavefront tile
-            int64_t brow;
-            if constexpr (GATED) {
-              int col = n0 + wn * 64 + (local & 63);
-              col = col < p.N ? col : p.N - 1;
-              const int half = local >> 6;
-              brow = p.interleaved ? 2 * col + half : half * p.N + col;
-            } else {
-              const int col = n0 + wn * 128 + local;
-              brow = col < p.N ? col : p.N - 1;
-            }
-            v[i] += El::ld(bias[e * p.bias_stride_e + brow]);
-          }
+          for (int i = 0; i < 4; ++i) v[i] += El::ld(bias[e * p.bias_stride_e + wrow_of(fn, g, i)]);
         }
         if (p.mul_weight) {
 #pragma unroll
@@ -721,8 +785,8 @@ __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, i
 
 template <typename Mma, int FMC, bool GATED>
 __device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, char* smem, int nk,
-                                         int e, int n0, int wn, int lane, int my_tok, float my_rw,
-                                         int* s_tok_all, float* s_rw_all, const float* s_rw, char* epi) {
+                                         int e, int n0, int wn, int wm, int lane, int my_tok, float my_rw,
+                                         float my_as, int* s_tok_all, float* s_rw_all, char* epi) {
   using El = typename Mma::El;
   f32x16 acc[4][4];
 #pragma unroll
@@ -735,9 +799,12 @@ __device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, c
   bare_barrier();  // every wavefront is done reading the ring before it is reused
   s_tok_all[threadIdx.x] = my_tok;
   s_rw_all[threadIdx.x] = my_rw;  // requested before the main loop, needed only now
+  s_rw_all[kBigBM + threadIdx.x] = my_as;
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   bare_barrier();
-  if constexpr (FMC > 0) big_park<El, FMC, GATED>(p, e, n0, wn, lane >> 5, lane & 31, s_rw, epi, acc);
+  if constexpr (FMC > 0)
+    big_park<El, FMC, GATED, Mma::kEs == 1>(p, e, n0, wn, lane >> 5, lane & 31, s_rw_all + wm * 128,
+                                            s_rw_all + kBigBM + wm * 128, epi, acc);
 }
 
 template <typename Mma, bool GATED>
@@ -781,14 +848,16 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   __syncthreads();
   const int nvalid = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
   if (nvalid == 0) return;
-  float my_rw = 1.f;
+  float my_rw = 1.f, my_as = 1.f;
   if (p.mul_weight) my_rw = my_tok < p.numel ? p.topk_w[my_tok] : 0.f;
+  if (p.a_scale && my_tok < p.numel) my_as = p.a_scale[p.a_by_slot ? my_slot : my_tok / p.top_k];
+  constexpr int ES = Mma::kEs, CH = Mma::kBigChunks;
 
   BigCtx c;
   const int ld_row = tid >> 3;                        // row inside a 32-row load group
   const int ld_chunk = (tid & 7) ^ ((tid >> 4) & 7);  // logical chunk this lane fetches
   c.a_base = static_cast<const char*>(p.a);
-  c.w_base = static_cast<const char*>(p.w) + static_cast<int64_t>(e) * p.w_stride_e * 2;
+  c.w_base = static_cast<const char*>(p.w) + static_cast<int64_t>(e) * p.w_stride_e * ES;
   const int a_groups = (nvalid + 31) >> 5;  // 32-row token groups that hold real slots
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -801,7 +870,7 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
       const int tok = s_tok[ld_row + 32 * gi];
       src = tok < p.numel ? tok / p.top_k : 0;
     }
-    c.a_off[i] = static_cast<uint32_t>((src * p.lda + ld_chunk * 8) * 2);
+    c.a_off[i] = static_cast<uint32_t>(src * p.lda * ES + ld_chunk * 16);
     const int rr = ld_row + 32 * i;
     int64_t wrow;
     if constexpr (GATED) {
@@ -813,11 +882,13 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
       const int n = n0 + rr;
       wrow = n < p.N ? n : p.N - 1;
     }
-    c.w_off[i] = static_cast<uint32_t>((wrow * p.w_stride_n + ld_chunk * 8) * 2);
+    c.w_off[i] = static_cast<uint32_t>(wrow * p.w_stride_n * ES + ld_chunk * 16);
   }
   c.dma_lds = __builtin_amdgcn_readfirstlane(lds_offset_of(smem) + wave * 1024);
+  // chunk ch of MFMA step kk: lane half lhi owns the K elements of chunks CH * (2 kk + lhi) .. + CH - 1
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) c.rd_k[kk] = l32 * kBigRowBytes + (((2 * kk + lhi) ^ ((l32 >> 1) & 7)) << 4);
+  for (int q = 0; q < 4; ++q)
+    c.rd_k[q] = l32 * kBigRowBytes + (((CH * (2 * (q / CH) + lhi) + q % CH) ^ ((l32 >> 1) & 7)) << 4);
   c.x_row = wm * 128 * kBigRowBytes;
 #pragma unroll
   for (int fn = 0; fn < 4; ++fn) {
@@ -828,18 +899,18 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
       r = wn * 128 + fn * 32;
     c.w_row[fn] = r * kBigRowBytes;
   }
-  const int nk = p.Kd / kBigBK;
+  const int nk = p.Kd / (kBigRowBytes / ES);
   const int slot0 = mb * kBigBM + wm * 128;
   char* epi = smem + wave * kEpiWaveBytes;
   [[maybe_unused]] const unsigned long long t_pro = MOE_TRACE_NOW();
   const int rows = min(128, max(0, nvalid - wm * 128));  // real slots of this wavefront
   __syncthreads();  // s_tok sits inside the ring: everyone has read it before any DMA may land there
   switch ((rows + 31) >> 5) {
-    case 0: big_wave<Mma, 0, GATED>(p, c, smem, nk, e, n0, wn, lane, my_tok, my_rw, s_tok, s_rw_all, s_rw_all + wm * 128, epi); break;
-    case 1: big_wave<Mma, 1, GATED>(p, c, smem, nk, e, n0, wn, lane, my_tok, my_rw, s_tok, s_rw_all, s_rw_all + wm * 128, epi); break;
-    case 2: big_wave<Mma, 2, GATED>(p, c, smem, nk, e, n0, wn, lane, my_tok, my_rw, s_tok, s_rw_all, s_rw_all + wm * 128, epi); break;
-    case 3: big_wave<Mma, 3, GATED>(p, c, smem, nk, e, n0, wn, lane, my_tok, my_rw, s_tok, s_rw_all, s_rw_all + wm * 128, epi); break;
-    default: big_wave<Mma, 4, GATED>(p, c, smem, nk, e, n0, wn, lane, my_tok, my_rw, s_tok, s_rw_all, s_rw_all + wm * 128, epi); break;
+    case 0: big_wave<Mma, 0, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, s_tok, s_rw_all, epi); break;
+    case 1: big_wave<Mma, 1, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, s_tok, s_rw_all, epi); break;
+    case 2: big_wave<Mma, 2, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, s_tok, s_rw_all, epi); break;
+    case 3: big_wave<Mma, 3, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, s_tok, s_rw_all, epi); break;
+    default: big_wave<Mma, 4, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, s_tok, s_rw_all, epi); break;
   }
   [[maybe_unused]] const unsigned long long t_main = MOE_TRACE_NOW();
   if constexpr (GATED) {
@@ -1156,6 +1227,13 @@ template <typename Mma, bool GATED>
 int launch_bm(GemmParams& p, int block_size, int64_t sorted_cap, hipStream_t s) {
   p.align_bs = block_size;
   p.m_major = 0;
+  if constexpr (Mma::kEs == 1) {
+    // a large-tile K step is 128 bytes per row: 128 e4m3 elements
+    if (block_size % 256 == 0 && p.Kd % kBigRowBytes == 0) {
+      p.m_major = 1;
+      return launch_big<MmaE4M3Big<typename Mma::El>, GATED>(p, sorted_cap, s);
+    }
+  }
   if constexpr (Mma::kEs == 2) {
     if (block_size % 256 == 0 && p.Kd % kBigBK == 0) {
       p.m_major = 1;  // a token block is reused by all its n-tiles through one L2
@@ -1192,7 +1270,7 @@ MOE_EXPORT int moe_preferred_block_size(int M, int E, int K, int act_dtype, int 
   (void)act_dtype;
   if (E < 1) return 64;
   const int64_t avg = static_cast<int64_t>(M) * K / E;  // routed rows per expert
-  if (avg >= 256 && weight_dtype != MOE_E4M3) return 256;  // no large-tile e4m3 kernel yet
+  if (avg >= 256) return 256;
   if (avg >= 96) return 128;
   if (avg >= 24) return 64;
   return 32;

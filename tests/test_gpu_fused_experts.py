@@ -242,6 +242,26 @@ def test_fused_experts_fp8_against_dequantised_oracle(moe, oracle, dev, E, H, I,
     assert (out.float().cpu() - full).abs().max() < 0.25 * full.abs().max() + 0.05
 
 
+@pytest.mark.parametrize("bm", [32, 64, 128, 256, 512])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fp8_every_block_size_kernel(moe, oracle, dev, bm, dtype, monkeypatch):
+    """Blocks of 256 slots run the large-tile e4m3 kernel (K = 64 MFMA steps),
+    smaller ones the register-staged kernels; both must agree with the oracle
+    that rounds where the kernels store."""
+    x, w13, w2, logits = _layer(16, 512, 256, 700, 4, 77, dtype)
+    tw, ids, _ = oracle.topk_softmax(logits, 4, renormalize=True)
+    w13q, w13s, w2q, w2s = moe.quantize_expert_weights(w13.to(dev), w2.to(dev))
+    monkeypatch.setattr(moe.fused_moe, "try_get_optimal_moe_config",
+                        lambda *a, **k: {"BLOCK_SIZE_M": bm})
+    out = moe.fused_experts(x.to(dev), w13q, w2q, None, None, tw.to(dev), ids.to(dev),
+                            per_channel_quant=True, w1_scale=w13s, w2_scale=w2s)
+    torch.cuda.synchronize()
+    mirrored = oracle.fused_experts_fp8_ref(x, w13q.view(torch.uint8).cpu(), w13s.cpu(),
+                                            w2q.view(torch.uint8).cpu(), w2s.cpu(), tw, ids,
+                                            mirror_rounding=True)
+    _close(out, mirrored, rtol=2e-2, atol=0.03 * mirrored.abs().max().item())
+
+
 def test_fp8_layered_prefill_batch_sampled_rows(moe, oracle, dev):
     """Config 5: the 8192+256 batch with e4m3 weights and per-token e4m3
     activations; sampled rows against the fp32 dequantised oracle."""
