@@ -200,23 +200,35 @@ __global__ __launch_bounds__(kScanThreads) void align_scan_kernel(
   __shared__ int s_cum[kMaxExperts + 1];
   __shared__ int s_tot[kMaxExperts];
   __shared__ int s_wave_tot[kScanWaves + 1];
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  // per expert: exclusive prefix of its counts over segments (in place)
-  for (int e = wave; e < E; e += kScanWaves) {
-    int running = 0;
-    for (int s0 = 0; s0 < nseg; s0 += kWave) {
-      const int s = s0 + lane;
-      const int c = s < nseg ? seg_cnt[static_cast<size_t>(s) * E + e] : 0;
-      int inc = c;
-#pragma unroll
-      for (int d = 1; d < kWave; d *= 2) {
-        int o = __shfl_up(inc, d, kWave);
-        if (lane >= d) inc += o;
-      }
-      if (s < nseg) seg_cnt[static_cast<size_t>(s) * E + e] = running + inc - c;
-      running += __shfl(inc, kWave - 1, kWave);
+  // per expert: exclusive prefix of its counts over segments (in place).
+  // Thread t works on expert t % E and on the (t / E)-th range of segments, so
+  // that a wavefront reads 64 consecutive experts of one segment (one 256-byte
+  // line; indexing the lanes by segment would touch 64 lines per load).
+  __shared__ int s_part[kScanThreads];
+  const int R = kScanThreads / E;                 // segment ranges (E <= kScanThreads)
+  const int L = (nseg + R - 1) / R;               // segments per range
+  const int e = threadIdx.x % E, r = threadIdx.x / E;
+  const bool active = r < R;
+  const int sbeg = r * L, send = min(nseg, sbeg + L);
+  int sum = 0;
+  if (active)
+    for (int sg = sbeg; sg < send; ++sg) sum += seg_cnt[static_cast<size_t>(sg) * E + e];
+  if (active) s_part[r * E + e] = sum;
+  __syncthreads();
+  if (active) {
+    int running = 0, total = 0;
+    for (int q = 0; q < R; ++q) {
+      const int v = s_part[q * E + e];
+      if (q < r) running += v;
+      total += v;
     }
-    if (lane == 0) s_tot[e] = running;
+    if (r == 0) s_tot[e] = total;
+    for (int sg = sbeg; sg < send; ++sg) {
+      const size_t at = static_cast<size_t>(sg) * E + e;
+      const int c = seg_cnt[at];
+      seg_cnt[at] = running;
+      running += c;
+    }
   }
   __syncthreads();
   int padded = 0;
