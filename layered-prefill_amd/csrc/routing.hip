@@ -74,8 +74,15 @@ __global__ __launch_bounds__(kWave* kWavesPerBlock) void topk_softmax_pow2_kerne
     v[i] = p < kFltMin ? 0.f : p;
   }
 
+  // Up to kRegK winners stay in registers until the row is done, so that the
+  // renormalised weights are written once (reading the stored weights back
+  // would wait for the stores to complete).
+  constexpr int kRegK = 16;
   float wsum = 0.f;
-  for (int k = 0; k < K; ++k) {
+  float bw[kRegK];
+#pragma unroll
+  for (int k = 0; k < kRegK; ++k) bw[k] = 0.f;
+  auto round = [&](int k, float& best_out) {
     float best = v[0];
     int bidx = t * EPL;
 #pragma unroll
@@ -91,22 +98,38 @@ __global__ __launch_bounds__(kWave* kWavesPerBlock) void topk_softmax_pow2_kerne
     }
     if (live && t == 0) {
       const size_t o = static_cast<size_t>(row) * K + k;
-      topk_w[o] = best;
       topk_ids[o] = bidx;
       tok_exp_idx[o] = k * T + row;
     }
     wsum += best;
+    best_out = best;
     // blank the winner in the lane that holds it
     const int owner = (bidx / EPL) % TPR;
     const int slot = (bidx / (EPL * TPR)) * EPL + (bidx % EPL);
 #pragma unroll
     for (int i = 0; i < VPT; ++i)
       if (t == owner && i == slot) v[i] = -10000.f;
-  }
-  if (renormalize && live && t == 0) {
+  };
+  if (K <= kRegK) {
+#pragma unroll
+    for (int k = 0; k < kRegK; ++k)
+      if (k < K) round(k, bw[k]);
+    if (live && t == 0) {
+#pragma unroll
+      for (int k = 0; k < kRegK; ++k)
+        if (k < K) topk_w[static_cast<size_t>(row) * K + k] = renormalize ? bw[k] / wsum : bw[k];
+    }
+  } else {
     for (int k = 0; k < K; ++k) {
-      const size_t o = static_cast<size_t>(row) * K + k;
-      topk_w[o] = topk_w[o] / wsum;
+      float best;
+      round(k, best);
+      if (live && t == 0) topk_w[static_cast<size_t>(row) * K + k] = best;
+    }
+    if (renormalize && live && t == 0) {
+      for (int k = 0; k < K; ++k) {
+        const size_t o = static_cast<size_t>(row) * K + k;
+        topk_w[o] = topk_w[o] / wsum;
+      }
     }
   }
 }
