@@ -33,8 +33,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs (profiles/hbm_traffic_gate_up_kernels.txt): fetch + write bytes.
-MEASURED_TRAFFIC_BYTES = {"layered_8192p_256d": 1693171712 + 144224256,
-                          "decode_256": 518821888 + 3155968}
+MEASURED_TRAFFIC_BYTES = {"layered_8192p_256d": 1764225024 + 150441984,
+                          "decode_256": 570650624 + 3343360}
 
 
 def _events(n):
@@ -276,7 +276,7 @@ def main() -> int:
         # dominant kernel: gate-up grouped GEMM, 4*T*K*H*I algorithmic flops
         k_flops = 4 * main_layer.T * shape.top_k * shape.hidden * shape.intermediate
         ach = k_flops / (stages["gate_up_gemm_act"] * 1e-3) / 1e12
-        roofline = {"bound": "mfma", "kernel": "grouped_gemm_kernel<gate-up, SiLU*up epilogue>",
+        roofline = {"bound": "mfma", "kernel": "big_gemm_kernel<MmaBF16, gated> (gate-up GEMM, SiLU*up epilogue)",
                     "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(ach / PEAK_BF16_TFLOPS, 4),
                     "kernel_ms": round(stages["gate_up_gemm_act"], 4),
@@ -286,7 +286,7 @@ def main() -> int:
         # dominant kernel: gate-up grouped GEMM streaming 2*H*I weights per active expert
         k_bytes = n_active * 2 * shape.hidden * shape.intermediate * 2 + main_layer.T * shape.hidden * 2
         ach = k_bytes / (stages["gate_up_gemm_act"] * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "kernel": "grouped_gemm_kernel<gate-up, SiLU*up epilogue>",
+        roofline = {"bound": "hbm", "kernel": "stream_gemm_kernel<MmaBF16, gated> (gate-up GEMM, SiLU*up epilogue)",
                     "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                     "frac": round(ach / PEAK_HBM_GBS, 4),
                     "kernel_ms": round(stages["gate_up_gemm_act"], 4),
