@@ -98,6 +98,27 @@ def time_steps(layer: Layer, steps: int, warmup: int):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
+def time_steps_flushed(layer: Layer, steps: int):
+    """Per-step event timing with L2 and the 256 MB memory-side cache overwritten
+    between steps (a 1 GiB fill), so that no expert weight of the previous step
+    is served from a cache.  Returns (median, p10, p90) in ms."""
+    flush = torch.empty(1 << 30, dtype=torch.uint8, device=layer.dev)
+    times = []
+    for i in range(steps + 3):
+        flush.fill_(i & 0xff)
+        ev = _events(2)
+        ev[0].record()
+        layer.step()
+        ev[1].record()
+        torch.cuda.synchronize()
+        if i >= 3:
+            times.append(ev[0].elapsed_time(ev[1]))
+    del flush
+    times.sort()
+    pick = lambda q: times[min(len(times) - 1, int(q * len(times)))]
+    return pick(0.5), pick(0.1), pick(0.9)
+
+
 def time_graph_replays(layer: Layer, steps: int, warmup: int):
     """The same step recorded once into a HIP graph and replayed: what a serving
     loop that captures its decode iteration pays (the reference runs this layer
@@ -343,6 +364,10 @@ def main() -> int:
                          "hbm_gbs": round(dgbs, 1), "frac_of_hbm_peak": round(dgbs / PEAK_HBM_GBS, 4),
                          "active_experts": dact, "block_size_m": dec.bm,
                          "stage_ms": {k: round(v, 4) for k, v in dstages.items()}}
+        fmed, fp10, fp90 = time_steps_flushed(dec, 30)
+        out["decode"]["cache_flushed"] = {"ms_median": round(fmed, 4), "ms_p10": round(fp10, 4),
+                                          "ms_p90": round(fp90, 4),
+                                          "hbm_gbs": round(dbytes / (fmed * 1e-3) / 1e9, 1)}
         if not a.no_graph:
             gms, gerr = time_graph_replays(dec, max(a.steps, 50), max(a.warmup, 10))
             ggbs = dbytes / (gms * 1e-3) / 1e9

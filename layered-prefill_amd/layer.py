@@ -1,9 +1,11 @@
 """``FusedMoE`` module with the interface of the reference's
 ``nanovllm/layers/fused_moe.py`` (types at :23-57, UnquantizedFusedMoEMethod at
-:108-216, FusedMoE.__init__/select_experts/forward at :218-320,693-787), on top
-of the HIP expert path.  TP=1 only: the reference's optional all-reduce
-(:746-748,782-785) belongs to its custom_all_reduce layer and is not part of
-this build, so ``reduce_results=True`` with more than one rank raises.
+:108-216, FusedMoE.__init__/select_experts/forward at :218-320,693-787, the
+checkpoint loader at :330-658 and ``make_expert_params_mapping`` at :789-821),
+on top of the HIP expert path.  TP=1 only at run time: the reference's optional
+all-reduce (:746-748,782-785) belongs to its custom_all_reduce layer and is not
+part of this build, so ``reduce_results=True`` with more than one rank raises.
+The loader does slice for a tensor-parallel rank, as the reference's does.
 """
 from __future__ import annotations
 
@@ -104,8 +106,46 @@ class UnquantizedFusedMoEMethod:
             global_num_experts=global_num_experts, expert_map=expert_map)
 
 
+class Fp8E4M3FusedMoEMethod(UnquantizedFusedMoEMethod):
+    """Per-output-channel e4m3 weights with dynamic per-token e4m3 activations.
+    No counterpart in the reference (its ``fused_experts`` asserts the scale
+    arguments are None, nanovllm/layers/for_moe/fused_moe.py:248-249); this is
+    where the one-time weight quantisation lives.  Weights are created and
+    loaded in ``params_dtype`` exactly like the unquantised method;
+    ``process_weights_after_loading`` then replaces them by e4m3 codes and adds
+    ``w13_weight_scale [E, 2I]`` / ``w2_weight_scale [E, H]`` (fp32)."""
+
+    def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
+        from .fused_moe import quantize_expert_weights
+        w13q, w13s, w2q, w2s = quantize_expert_weights(layer.w13_weight.data, layer.w2_weight.data)
+        layer.w13_weight = torch.nn.Parameter(w13q, requires_grad=False)
+        layer.w2_weight = torch.nn.Parameter(w2q, requires_grad=False)
+        layer.register_parameter("w13_weight_scale", torch.nn.Parameter(w13s, requires_grad=False))
+        layer.register_parameter("w2_weight_scale", torch.nn.Parameter(w2s, requires_grad=False))
+
+    def apply(self, layer: torch.nn.Module, x: torch.Tensor, router_logits: torch.Tensor,
+              top_k: int, renormalize: bool, activation: str = "silu",
+              apply_router_weight_on_input: bool = False, global_num_experts: int = -1,
+              expert_map: Optional[torch.Tensor] = None,
+              custom_routing_function: Optional[Callable] = None, **unused) -> torch.Tensor:
+        if not hasattr(layer, "w13_weight_scale"):
+            raise RuntimeError("Fp8E4M3FusedMoEMethod.apply before process_weights_after_loading")
+        topk_weights, topk_ids = FusedMoE.select_experts(
+            hidden_states=x, router_logits=router_logits, use_grouped_topk=False, top_k=top_k,
+            renormalize=renormalize, custom_routing_function=custom_routing_function,
+            indices_type=self.topk_indices_dtype)
+        return self.fused_experts(
+            hidden_states=x, w1=layer.w13_weight, w2=layer.w2_weight,
+            w1_bias=layer.w13_bias if hasattr(layer, "w13_bias") else None,
+            w2_bias=layer.w2_bias if hasattr(layer, "w2_bias") else None,
+            topk_weights=topk_weights, topk_ids=topk_ids, inplace=True, activation=activation,
+            apply_router_weight_on_input=apply_router_weight_on_input, per_channel_quant=True,
+            global_num_experts=global_num_experts, expert_map=expert_map,
+            w1_scale=layer.w13_weight_scale, w2_scale=layer.w2_weight_scale)
+
+
 class FusedMoE(torch.nn.Module):
-    """nanovllm/layers/fused_moe.py:218-320,693-787."""
+    """nanovllm/layers/fused_moe.py:218-320,330-658,693-821."""
 
     def __init__(self, num_experts: int, top_k: int, hidden_size: int, intermediate_size: int,
                  params_dtype: Optional[torch.dtype] = None, reduce_results: bool = False,
@@ -117,7 +157,8 @@ class FusedMoE(torch.nn.Module):
                  scoring_func: str = "softmax",
                  e_score_correction_bias: Optional[torch.Tensor] = None,
                  apply_router_weight_on_input: bool = False, activation: str = "silu",
-                 num_redundant_experts: int = 0, has_bias: bool = False):
+                 num_redundant_experts: int = 0, has_bias: bool = False,
+                 quantization: Optional[str] = None):
         super().__init__()
         if params_dtype is None:
             params_dtype = torch.get_default_dtype()
@@ -152,11 +193,130 @@ class FusedMoE(torch.nn.Module):
             num_local_experts=self.local_num_experts,
             moe_parallel_config=self.moe_parallel_config, in_dtype=params_dtype,
             quant_dtype=params_dtype, max_num_tokens=256)
-        self.quant_method = UnquantizedFusedMoEMethod(self.moe_config)
+        # `quantization` has no counterpart in the reference constructor (it only
+        # builds the unquantised method, :300-304); "fp8_e4m3" selects the e4m3 path
+        if quantization is None:
+            self.quant_method = UnquantizedFusedMoEMethod(self.moe_config)
+        elif quantization == "fp8_e4m3":
+            self.quant_method = Fp8E4M3FusedMoEMethod(self.moe_config)
+        else:
+            raise ValueError(f"unsupported quantization {quantization!r}")
         self.quant_method.create_weights(
             layer=self, num_experts=self.local_num_experts, hidden_size=hidden_size,
             intermediate_size_per_partition=self.intermediate_size_per_partition,
-            params_dtype=params_dtype, has_bias=has_bias)
+            params_dtype=params_dtype, has_bias=has_bias, weight_loader=self.weight_loader)
+
+    # ------------------------------------------------------------------ checkpoint loading
+    _SHARDED_DIM = {"w1": 0, "w2": 1, "w3": 0, "w13": 1}
+
+    def _tp_slice(self, tensor: torch.Tensor, dim: int, size: int) -> torch.Tensor:
+        """This rank's `size` entries of `tensor` along `dim`."""
+        return tensor.narrow(dim, size * self.tp_rank, size)
+
+    def _load_w13(self, expert_data: torch.Tensor, shard_dim: int, shard_id: str,
+                  loaded_weight: torch.Tensor) -> None:
+        # gate_proj fills the first half of w13 along shard_dim, up_proj the second
+        # (nanovllm/layers/fused_moe.py:398-414); column-parallel over the rank
+        half = expert_data.shape[shard_dim] // 2
+        src = self._tp_slice(loaded_weight, shard_dim, half)
+        expert_data.narrow(shard_dim, 0 if shard_id == "w1" else half, half).copy_(src)
+
+    def _load_w2(self, expert_data: torch.Tensor, shard_dim: int,
+                 loaded_weight: torch.Tensor) -> None:
+        # down_proj is row-parallel: the rank keeps its slice of the input dimension
+        # (nanovllm/layers/fused_moe.py:416-432)
+        expert_data.copy_(self._tp_slice(loaded_weight, shard_dim, expert_data.shape[shard_dim]))
+
+    def _load_matrix(self, shard_id: str, shard_dim: int, expert_data: torch.Tensor,
+                     loaded_weight: torch.Tensor) -> None:
+        if expert_data.ndim != loaded_weight.ndim:
+            loaded_weight = loaded_weight.reshape(*loaded_weight.shape[:-2], -1)
+        if shard_id == "w2":
+            self._load_w2(expert_data, shard_dim, loaded_weight)
+        elif shard_id in ("w1", "w3"):
+            self._load_w13(expert_data, shard_dim, shard_id, loaded_weight)
+        else:  # "w13": gate and up already merged in the checkpoint
+            size = expert_data.shape[1]
+            expert_data.narrow(1, 0, size).copy_(loaded_weight.narrow(1, size * self.tp_rank, size))
+
+    def weight_loader(self, param: torch.nn.Parameter, loaded_weight: torch.Tensor,
+                      weight_name: str, shard_id: str, expert_id: int,
+                      return_success: bool = False) -> Optional[bool]:
+        """Copies one checkpoint tensor into its place in ``w13_weight`` /
+        ``w2_weight`` (or a bias / per-channel scale), same contract as
+        nanovllm/layers/fused_moe.py:472-658: ``shard_id`` is ``w1`` (gate_proj),
+        ``w3`` (up_proj), ``w2`` (down_proj), ``w13`` (merged gate_up) or ``all``
+        (all experts in one tensor); tensors are sliced for this TP rank.
+        Checkpoint formats the reference routes to other quantisation methods
+        (GGUF, g_idx, ModelOpt, group/block/tensor scales, input scales) are
+        rejected: no such method exists on this path."""
+        ok = True if return_success else None
+        if shard_id == "all":
+            if "bias" in weight_name:
+                param.data.copy_(loaded_weight)
+            else:
+                param.data.copy_(loaded_weight.reshape(*param.data.shape[:-1], -1))
+            return ok
+        if self.expert_map is not None:
+            expert_id = int(self.expert_map[expert_id])
+            if expert_id == -1:
+                return False if return_success else None
+        if shard_id not in self._SHARDED_DIM:
+            raise ValueError(f"shard_id must be ['w1','w2','w3', 'all'] but got {shard_id}.")
+        for marker in ("input_scale", "g_idx", "weight_shape", "zero", "offset"):
+            if marker in weight_name:
+                raise ValueError(f"{weight_name}: '{marker}' tensors belong to quantisation "
+                                 "methods this layer does not have")
+        shard_dim = self._SHARDED_DIM[shard_id]
+        if getattr(param, "is_transposed", False):
+            shard_dim = 1 - shard_dim
+        full_load = loaded_weight.dim() == 3 or "bias" in weight_name
+        if full_load:
+            shard_dim += 1
+        expert_data = param.data if full_load else param.data[expert_id]
+        if "scale" in weight_name:
+            # per-output-channel weight scales of the e4m3 method: a vector per expert
+            if shard_id == "w2":
+                expert_data.copy_(loaded_weight)
+            else:
+                self._load_w13(expert_data, shard_dim, shard_id, loaded_weight)
+            return ok
+        if "weight" in weight_name:
+            self._load_matrix(shard_id, shard_dim, expert_data, loaded_weight)
+            return ok
+        if "bias" in weight_name:
+            if shard_id == "w2":
+                # the down bias is added once: only rank 0 keeps it
+                if self.tp_rank == 0:
+                    expert_data.copy_(loaded_weight)
+                else:
+                    expert_data.zero_()
+            else:
+                n = loaded_weight.size(-1) // self.tp_size
+                expert_data.copy_(loaded_weight.narrow(-1, self.tp_rank * n, n))
+            return ok
+        raise ValueError(f"Unrecognized weight_name {weight_name}.")
+
+    @classmethod
+    def make_expert_params_mapping(cls, ckpt_gate_proj_name: str, ckpt_down_proj_name: str,
+                                   ckpt_up_proj_name: str, num_experts: int,
+                                   num_redundant_experts: int = 0) -> list:
+        """``(param_name, weight_name, expert_id, shard_id)`` for every physical
+        expert and projection (nanovllm/layers/fused_moe.py:789-821); redundant
+        experts replay the logical ones round-robin."""
+        logical = list(range(num_experts)) + [i % num_experts for i in range(num_redundant_experts)]
+        mapping = []
+        for expert_id, logical_id in enumerate(logical):
+            for shard_id, name in (("w1", ckpt_gate_proj_name), ("w2", ckpt_down_proj_name),
+                                   ("w3", ckpt_up_proj_name)):
+                param = "experts.w13_" if name in (ckpt_gate_proj_name, ckpt_up_proj_name) else "experts.w2_"
+                mapping.append((param, f"experts.{logical_id}.{name}.", expert_id, shard_id))
+        return mapping
+
+    def process_weights_after_loading(self) -> None:
+        hook = getattr(self.quant_method, "process_weights_after_loading", None)
+        if hook is not None:
+            hook(self)
 
     @property
     def tp_size(self) -> int:
