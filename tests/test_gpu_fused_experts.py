@@ -1,5 +1,7 @@
 """GPU parity of the expert MLP (grouped GEMMs, fused activation, combine) and
 of the stand-alone activation / combine ops against the CPU oracle."""
+import os
+
 import pytest
 import torch
 
@@ -310,3 +312,52 @@ def test_layer_step_replays_from_a_hip_graph(moe, oracle, dev):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(static_out, want), f"replay {r} differs from the eager result"
+
+
+def _random_cases(n, seed):
+    import random
+    rnd = random.Random(seed)
+    cases = []
+    for i in range(n):
+        E = rnd.choice([1, 3, 8, 16, 40, 128])
+        K = rnd.choice([k for k in (1, 2, 4, 8) if k <= E])
+        H = 64 * rnd.randint(1, 8) if rnd.random() < 0.8 else 8 * rnd.randint(3, 40)
+        I = 64 * rnd.randint(1, 6) if rnd.random() < 0.7 else 8 * rnd.randint(2, 30)
+        T = rnd.choice([1, 2, 7, 33, 64, 100, 257, 700, 1500])
+        bm = rnd.choice([0, 0, 32, 64, 128, 256])
+        dtype = rnd.choice(["bf16", "bf16", "f16", "fp8"])
+        if dtype == "fp8":  # one-byte elements: rows are addressed in 16-byte chunks
+            H, I = max(16, H // 16 * 16), max(16, I // 16 * 16)
+        cases.append((i, E, K, H, I, T, bm, dtype))
+    return cases
+
+
+# MOE_FUZZ_N / MOE_FUZZ_SEED widen the sweep for a one-off run
+@pytest.mark.parametrize("case", _random_cases(int(os.environ.get("MOE_FUZZ_N", "36")),
+                                               int(os.environ.get("MOE_FUZZ_SEED", "20250"))),
+                         ids=lambda c: "-".join(map(str, c)))
+def test_random_shapes_all_kernels(moe, oracle, dev, case, monkeypatch):
+    """Seeded random layer shapes, token counts, block sizes and dtypes: every
+    dispatch branch (large-tile, streaming, register-staged; 16-bit and e4m3)
+    with ragged N / K, empty experts and single tokens, against the oracle that
+    rounds where the kernels store."""
+    i, E, K, H, I, T, bm, dt = case
+    dtype = torch.float16 if dt == "f16" else torch.bfloat16
+    x, w13, w2, logits = _layer(E, H, I, T, K, 1000 + i, dtype)
+    tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
+    if bm:
+        monkeypatch.setattr(moe.fused_moe, "try_get_optimal_moe_config",
+                            lambda *a, **k: {"BLOCK_SIZE_M": bm})
+    d = lambda t: t.to(dev)
+    if dt == "fp8":
+        w13q, w13s, w2q, w2s = moe.quantize_expert_weights(d(w13), d(w2))
+        out = moe.fused_experts(d(x), w13q, w2q, None, None, d(tw), d(ids), per_channel_quant=True,
+                                w1_scale=w13s, w2_scale=w2s)
+        ref = oracle.fused_experts_fp8_ref(x, w13q.view(torch.uint8).cpu(), w13s.cpu(),
+                                           w2q.view(torch.uint8).cpu(), w2s.cpu(), tw, ids,
+                                           mirror_rounding=True)
+        _close(out, ref, rtol=2e-2, atol=0.03 * ref.abs().max().item() + 1e-6)
+    else:
+        out = moe.fused_experts(d(x), d(w13), d(w2), None, None, d(tw), d(ids))
+        ref = oracle.fused_experts_ref(x, w13, w2, tw, ids, mirror_rounding=True)
+        _close(out, ref, rtol=1.6e-2, atol=2e-3 + 4e-3 * ref.abs().max().item())
