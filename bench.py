@@ -146,6 +146,35 @@ def time_graph_replays(layer: Layer, steps: int, warmup: int):
     return ms, float((out.float() - eager).abs().max())
 
 
+def time_router_gate(moe, layer: Layer, steps: int):
+    """Router gate ahead of the measured path (SURVEY 8f-2 of the scope table is
+    the fused form): gate linear + fused_topk as two steps, as the reference runs
+    them (nanovllm/models/qwen3_moe.py:93-104,113), against the one-kernel
+    fused_gate_topk.  Microseconds per call, events around `steps` calls."""
+    s = layer.shape
+    g = torch.Generator().manual_seed(99)
+    wg = (torch.randn(s.experts, s.hidden, generator=g) * 0.02).to(layer.x.dtype).to(layer.dev)
+
+    def two_step():
+        return moe.fused_topk(layer.x, torch.nn.functional.linear(layer.x, wg), s.top_k, True)
+
+    def fused():
+        return moe.fused_gate_topk(layer.x, wg, s.top_k, True)
+
+    out = {}
+    for name, fn in (("linear_then_topk_us", two_step), ("fused_gate_topk_us", fused)):
+        for _ in range(5):
+            fn()
+        ev = _events(2)
+        ev[0].record()
+        for _ in range(steps):
+            fn()
+        ev[1].record()
+        torch.cuda.synchronize()
+        out[name] = round(ev[0].elapsed_time(ev[1]) * 1e3 / steps, 2)
+    return out
+
+
 def time_stages(layer: Layer, steps: int):
     names = ["topk_softmax", "moe_align_block_size", "gate_up_gemm_act", "down_gemm_weighted",
              "topk_combine"]
@@ -327,6 +356,7 @@ def main() -> int:
         "roofline": roofline,
     }
 
+    out["router_gate"] = time_router_gate(moe, main_layer, 50)
     if compute_bound and a.chunk_mode != "off":
         out["chunk_amplification"] = chunk_amplification(moe, main_layer, max(2, a.steps // 10), a.chunk_mode)
     if compute_bound and not a.no_fp8:
@@ -364,6 +394,7 @@ def main() -> int:
                          "hbm_gbs": round(dgbs, 1), "frac_of_hbm_peak": round(dgbs / PEAK_HBM_GBS, 4),
                          "active_experts": dact, "block_size_m": dec.bm,
                          "stage_ms": {k: round(v, 4) for k, v in dstages.items()}}
+        out["decode"]["router_gate"] = time_router_gate(moe, dec, 100)
         fmed, fp10, fp90 = time_steps_flushed(dec, 30)
         out["decode"]["cache_flushed"] = {"ms_median": round(fmed, 4), "ms_p10": round(fp10, 4),
                                           "ms_p90": round(fp90, 4),

@@ -55,6 +55,19 @@ int moe_topk_softmax(const float* gating_output, float* topk_weights, int32_t* t
                      int32_t* token_expert_indices, int T, int E, int K, int renormalize,
                      void* stream);
 
+/* Router gate fused in front of `topk_softmax`: logits = x . gate_weight^T (the
+ * `ReplicatedLinear` gate of nanovllm/models/qwen3_moe.py:93-104 followed by the
+ * call at :113-118; nanovllm/layers/linear.py:53-60), rounded to the activation
+ * dtype as that layer's output is, then the routing of moe_topk_softmax.  The
+ * logits stay on chip; `logits_out` ([T, E] fp32, may be NULL) receives them when
+ * the caller wants to inspect them.  x [T, H] and gate_weight [E, H] are
+ * contiguous bf16 or fp16 (MoeDtype code), 16-byte aligned.  Supported shapes:
+ * E in {32, 64, 128}, H a multiple of 64; anything else returns
+ * MOE_ERR_UNSUPPORTED and the caller runs the gate and moe_topk_softmax apart. */
+int moe_gate_topk_softmax(const void* x, const void* gate_weight, int dtype, float* logits_out,
+                          float* topk_weights, int32_t* topk_ids, int32_t* token_expert_indices,
+                          int T, int H, int E, int K, int renormalize, void* stream);
+
 /* Replaces `moe_align_block_size` (csrc/moe_align_block_size_kernels.cu:239-291,
  * bound at csrc/ops.cpp:53-60,119-126).  `sorted_token_ids` (capacity
  * sorted_cap >= numel + E*(block_size-1)) receives, per expert in ascending

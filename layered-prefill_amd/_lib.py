@@ -26,7 +26,7 @@ EXPORTS = (
     "moe_last_error", "moe_abi_version", "moe_topk_softmax", "moe_align_workspace_bytes",
     "moe_align_block_size", "moe_silu_and_mul", "moe_swigluoai_and_mul", "moe_sum",
     "moe_fused_experts_workspace_bytes", "moe_fused_experts", "moe_preferred_block_size",
-    "moe_quant_rows_e4m3",
+    "moe_quant_rows_e4m3", "moe_gate_topk_softmax",
 )
 
 
@@ -68,6 +68,8 @@ def _declare(L: ctypes.CDLL) -> None:
     L.moe_abi_version.restype = i32
     L.moe_topk_softmax.restype = i32
     L.moe_topk_softmax.argtypes = [p, p, p, p, i32, i32, i32, i32, p]
+    L.moe_gate_topk_softmax.restype = i32
+    L.moe_gate_topk_softmax.argtypes = [p, p, i32, p, p, p, p, i32, i32, i32, i32, i32, p]
     L.moe_align_workspace_bytes.restype = i64
     L.moe_align_workspace_bytes.argtypes = [i64, i32]
     L.moe_align_block_size.restype = i32

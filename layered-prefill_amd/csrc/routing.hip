@@ -25,6 +25,149 @@ struct Pow2Geom {
 constexpr int kWavesPerBlock = 4;
 constexpr float kFltMin = 1.17549435e-38f;
 
+// Lane exchange for the order-independent reductions (max, argmax): partner at
+// distance M inside a row of TPR lanes.  Distances 1 and 2 are exact xor
+// butterflies (quad_perm); 4 and 8 use the mirror patterns of DPP, which pair
+// every lane with a lane of the other half of its 8- or 16-lane group: the same
+// thing once the lanes of each half already agree, which is why these
+// reductions run from distance 1 upwards.  DPP moves cost a few clocks; the
+// LDS-crossbar shuffle behind __shfl_xor costs ~100 and was most of a round.
+template <int M>
+__device__ __forceinline__ int lane_exchange(int v) {
+  if constexpr (M == 1) return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, true);        // quad_perm [1,0,3,2]
+  else if constexpr (M == 2) return __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, true);   // quad_perm [2,3,0,1]
+  else if constexpr (M == 4) return __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, true);  // row_half_mirror
+  else if constexpr (M == 8) return __builtin_amdgcn_update_dpp(0, v, 0x140, 0xf, 0xf, true);  // row_mirror
+  else return __shfl_xor(v, M, kWave);
+}
+template <int M>
+__device__ __forceinline__ float lane_exchange(float v) {
+  return __builtin_bit_cast(float, lane_exchange<M>(__builtin_bit_cast(int, v)));
+}
+
+template <int M, int TPR>
+__device__ __forceinline__ void max_level(float& mx) {
+  if constexpr (M < TPR) {
+    mx = fmaxf(mx, lane_exchange<M>(mx));
+    max_level<M * 2, TPR>(mx);
+  }
+}
+template <int M, int TPR>
+__device__ __forceinline__ void argmax_level(float& best, int& bidx) {
+  if constexpr (M < TPR) {
+    const float ov = lane_exchange<M>(best);
+    const int oi = lane_exchange<M>(bidx);
+    if (ov > best || (ov == best && oi < bidx)) { best = ov; bidx = oi; }
+    argmax_level<M * 2, TPR>(best, bidx);
+  }
+}
+
+// Softmax and K argmax rounds of one row spread over TPR lanes: lane t of the
+// row holds columns (i / EPL) * EPL * TPR + t * EPL + i % EPL in v[i].
+template <int E>
+__device__ __forceinline__ void route_row(float (&v)[Pow2Geom<E>::kVpt], int t, int row, bool live,
+                                          float* __restrict__ topk_w, int32_t* __restrict__ topk_ids,
+                                          int32_t* __restrict__ tok_exp_idx, int T, int K,
+                                          int renormalize) {
+  using G = Pow2Geom<E>;
+  constexpr int EPL = G::kEpl, VPT = G::kVpt, TPR = G::kTpr;
+  float mx = v[0];
+#pragma unroll
+  for (int i = 1; i < VPT; ++i) mx = fmaxf(mx, v[i]);
+  max_level<1, TPR>(mx);
+
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    v[i] = moe_expf(v[i] - mx);
+    sum += v[i];
+  }
+#pragma unroll
+  for (int m = TPR / 2; m > 0; m /= 2) sum += __shfl_xor(sum, m, kWave);
+  const float rinv = 1.f / sum;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    float p = v[i] * rinv;
+    v[i] = p < kFltMin ? 0.f : p;
+  }
+
+  // Up to kRegK winners stay in registers until the row is done (after the
+  // all-reduce every lane of the row knows them): the renormalised weights are
+  // then written once, and when the row has at least K lanes, lane k writes
+  // winner k, so a row's results leave as three short coalesced stores instead
+  // of three single-lane stores per round.
+  constexpr int kRegK = 16;
+  float wsum = 0.f;
+  float bw[kRegK];
+  int bi[kRegK];
+#pragma unroll
+  for (int k = 0; k < kRegK; ++k) { bw[k] = 0.f; bi[k] = 0; }
+  auto round = [&](float& best_out, int& bidx_out) {
+    float best = v[0];
+    int bidx = t * EPL;
+#pragma unroll
+    for (int i = 1; i < VPT; ++i) {
+      const int col = (i / EPL) * (EPL * TPR) + t * EPL + (i % EPL);
+      if (v[i] > best) { best = v[i]; bidx = col; }
+    }
+    argmax_level<1, TPR>(best, bidx);
+    wsum += best;
+    best_out = best;
+    bidx_out = bidx;
+    // blank the winner in the lane that holds it
+    const int owner = (bidx / EPL) % TPR;
+    const int slot = (bidx / (EPL * TPR)) * EPL + (bidx % EPL);
+#pragma unroll
+    for (int i = 0; i < VPT; ++i)
+      if (t == owner && i == slot) v[i] = -10000.f;
+  };
+  if (K <= kRegK) {
+#pragma unroll
+    for (int k = 0; k < kRegK; ++k)
+      if (k < K) round(bw[k], bi[k]);
+    if (K <= TPR) {
+      float my_w = 0.f;
+      int my_i = 0;
+#pragma unroll
+      for (int k = 0; k < kRegK; ++k)
+        if (t == k) { my_w = bw[k]; my_i = bi[k]; }
+      if (live && t < K) {
+        const size_t o = static_cast<size_t>(row) * K + t;
+        topk_w[o] = renormalize ? my_w / wsum : my_w;
+        topk_ids[o] = my_i;
+        tok_exp_idx[o] = t * T + row;
+      }
+    } else if (live && t == 0) {
+#pragma unroll
+      for (int k = 0; k < kRegK; ++k)
+        if (k < K) {
+          const size_t o = static_cast<size_t>(row) * K + k;
+          topk_w[o] = renormalize ? bw[k] / wsum : bw[k];
+          topk_ids[o] = bi[k];
+          tok_exp_idx[o] = k * T + row;
+        }
+    }
+  } else {
+    for (int k = 0; k < K; ++k) {
+      float best;
+      int bidx;
+      round(best, bidx);
+      if (live && t == 0) {
+        const size_t o = static_cast<size_t>(row) * K + k;
+        topk_w[o] = best;
+        topk_ids[o] = bidx;
+        tok_exp_idx[o] = k * T + row;
+      }
+    }
+    if (renormalize && live && t == 0) {
+      for (int k = 0; k < K; ++k) {
+        const size_t o = static_cast<size_t>(row) * K + k;
+        topk_w[o] = topk_w[o] / wsum;
+      }
+    }
+  }
+}
+
 template <int E>
 __global__ __launch_bounds__(kWave* kWavesPerBlock) void topk_softmax_pow2_kernel(
     const float* __restrict__ gating, float* __restrict__ topk_w, int32_t* __restrict__ topk_ids,
@@ -53,85 +196,200 @@ __global__ __launch_bounds__(kWave* kWavesPerBlock) void topk_softmax_pow2_kerne
     }
   }
 
-  float mx = v[0];
-#pragma unroll
-  for (int i = 1; i < VPT; ++i) mx = fmaxf(mx, v[i]);
-#pragma unroll
-  for (int m = TPR / 2; m > 0; m /= 2) mx = fmaxf(mx, __shfl_xor(mx, m, kWave));
+  route_row<E>(v, t, row, live, topk_w, topk_ids, tok_exp_idx, T, K, renormalize);
+}
 
-  float sum = 0.f;
-#pragma unroll
-  for (int i = 0; i < VPT; ++i) {
-    v[i] = moe_expf(v[i] - mx);
-    sum += v[i];
+// ---------------------------------------------------------------------------
+// Router gate fused in front: logits = x . Wg^T (the reference's ReplicatedLinear,
+// nanovllm/models/qwen3_moe.py:93-104, whose output has the activation dtype),
+// rounded to that dtype, then the same softmax / top-k as above, without the
+// logits ever leaving the CU.  A workgroup takes 32 tokens and all E experts
+// and walks K in units of 64 elements: the unit's 32 token rows and E gate rows
+// (128 bytes each) go global->LDS by DMA into a ring of four units, full
+// 128-byte lines per request (operands fetched straight into MFMA register
+// layout touch 64 different lines per wavefront load and ran 3x slower than the
+// separate GEMM + routing kernels).  Wavefront f multiplies expert fragment f
+// (MFMA 32x32x16, experts as the A operand, tokens as B); the rounded logits
+// are laid out in LDS as [token][expert] and routed from there with the lane
+// layout of the stand-alone kernel.
+// ---------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(8))) __bf16 gate_bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 gate_f16x8;
+typedef __attribute__((ext_vector_type(16))) float gate_f32x16;
+typedef __attribute__((address_space(3))) char gate_lds_char;
+
+template <typename El>
+__device__ __forceinline__ gate_f32x16 gate_mma(const uint4& a, const uint4& b, gate_f32x16 c);
+template <>
+__device__ __forceinline__ gate_f32x16 gate_mma<ElemBF16>(const uint4& a, const uint4& b, gate_f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(gate_bf16x8, a),
+                                                 __builtin_bit_cast(gate_bf16x8, b), c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ gate_f32x16 gate_mma<ElemF16>(const uint4& a, const uint4& b, gate_f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(gate_f16x8, a),
+                                                __builtin_bit_cast(gate_f16x8, b), c, 0, 0, 0);
+}
+
+// 16 bytes per lane from global memory straight into LDS at lds_wave_base + 16 * lane
+// (issued from assembly: the compiler would order every later LDS read behind it with vmcnt(0))
+__device__ __forceinline__ void gate_dma16(const char* base, uint32_t lane_byte_offset, uint32_t lds_wave_base) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2"
+      :
+      : "s"(lds_wave_base), "v"(lane_byte_offset), "s"(base)
+      : "memory");
+}
+
+constexpr int kGateTokens = 32, kGateRowBytes = 128;
+
+constexpr int kGateWaves = 16;  // wavefronts 0..3 stream and multiply; all sixteen route (two rows each)
+
+template <typename El, int E, int kGateRing>
+__global__ __launch_bounds__(kWave* kGateWaves) void gate_topk_softmax_kernel(
+    const typename El::S* __restrict__ x, const typename El::S* __restrict__ wg,
+    float* __restrict__ logits_out, float* __restrict__ topk_w, int32_t* __restrict__ topk_ids,
+    int32_t* __restrict__ tok_exp_idx, int T, int H, int K, int renormalize) {
+  using G = Pow2Geom<E>;
+  constexpr int NF = E / 32;                         // expert fragments = computing wavefronts
+  constexpr int WJ = E / 32;                         // gate-row requests per wavefront and unit
+  constexpr int kWBytes = E * kGateRowBytes;
+  constexpr int kUnitBytes = kWBytes + kGateTokens * kGateRowBytes;
+  constexpr int kDma = WJ + 1;                       // requests per wavefront and unit
+  static_assert(NF >= 1 && NF <= kWavesPerBlock, "one expert fragment per wavefront");
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int lane = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int l32 = lane & 31, lhi = lane >> 5;
+  const int t0 = blockIdx.x * kGateTokens;
+
+  // DMA: a request covers 8 rows x 128 bytes; lane / 8 is the row, lane % 8 the 16-byte chunk
+  // it lands in; chunk c of row r holds logical chunk c ^ ((r >> 1) & 7) (bank spreading)
+  const int q = lane >> 3;
+  uint32_t a_off, w_off[WJ];
+  {
+    const int rr = 8 * wave + q;
+    const int row = t0 + rr < T ? t0 + rr : T - 1;
+    a_off = static_cast<uint32_t>(static_cast<size_t>(row) * H * 2 + (((lane & 7) ^ ((rr >> 1) & 7)) << 4));
   }
 #pragma unroll
-  for (int m = TPR / 2; m > 0; m /= 2) sum += __shfl_xor(sum, m, kWave);
-  const float rinv = 1.f / sum;
-#pragma unroll
-  for (int i = 0; i < VPT; ++i) {
-    float p = v[i] * rinv;
-    v[i] = p < kFltMin ? 0.f : p;
+  for (int j = 0; j < WJ; ++j) {
+    const int rr = (E / 4) * wave + 8 * j + q;
+    w_off[j] = static_cast<uint32_t>(static_cast<size_t>(rr) * H * 2 + (((lane & 7) ^ ((rr >> 1) & 7)) << 4));
   }
-
-  // Up to kRegK winners stay in registers until the row is done, so that the
-  // renormalised weights are written once (reading the stored weights back
-  // would wait for the stores to complete).
-  constexpr int kRegK = 16;
-  float wsum = 0.f;
-  float bw[kRegK];
+  const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const gate_lds_char*)smem));
+  const uint32_t dma_w = __builtin_amdgcn_readfirstlane(lds0 + (E / 4) * wave * kGateRowBytes);
+  const uint32_t dma_a = __builtin_amdgcn_readfirstlane(lds0 + kWBytes + 8 * wave * kGateRowBytes);
+  const char* xb = reinterpret_cast<const char*>(x);
+  const char* wb = reinterpret_cast<const char*>(wg);
+  const bool worker = wave < kWavesPerBlock;  // the other wavefronts only keep the barriers company
+  auto issue = [&](int u) {
+    if (!worker) return;
+    const uint32_t ring = (u % kGateRing) * kUnitBytes;
+    gate_dma16(xb + u * kGateRowBytes, a_off, dma_a + ring);
 #pragma unroll
-  for (int k = 0; k < kRegK; ++k) bw[k] = 0.f;
-  auto round = [&](int k, float& best_out) {
-    float best = v[0];
-    int bidx = t * EPL;
-#pragma unroll
-    for (int i = 1; i < VPT; ++i) {
-      const int col = (i / EPL) * (EPL * TPR) + t * EPL + (i % EPL);
-      if (v[i] > best) { best = v[i]; bidx = col; }
-    }
-#pragma unroll
-    for (int m = TPR / 2; m > 0; m /= 2) {
-      float ov = __shfl_xor(best, m, kWave);
-      int oi = __shfl_xor(bidx, m, kWave);
-      if (ov > best || (ov == best && oi < bidx)) { best = ov; bidx = oi; }
-    }
-    if (live && t == 0) {
-      const size_t o = static_cast<size_t>(row) * K + k;
-      topk_ids[o] = bidx;
-      tok_exp_idx[o] = k * T + row;
-    }
-    wsum += best;
-    best_out = best;
-    // blank the winner in the lane that holds it
-    const int owner = (bidx / EPL) % TPR;
-    const int slot = (bidx / (EPL * TPR)) * EPL + (bidx % EPL);
-#pragma unroll
-    for (int i = 0; i < VPT; ++i)
-      if (t == owner && i == slot) v[i] = -10000.f;
+    for (int j = 0; j < WJ; ++j) gate_dma16(wb + u * kGateRowBytes, w_off[j], dma_w + ring + j * 1024);
   };
-  if (K <= kRegK) {
+  int rd_k[4];
 #pragma unroll
-    for (int k = 0; k < kRegK; ++k)
-      if (k < K) round(k, bw[k]);
-    if (live && t == 0) {
+  for (int kk = 0; kk < 4; ++kk) rd_k[kk] = l32 * kGateRowBytes + (((2 * kk + lhi) ^ ((l32 >> 1) & 7)) << 4);
+
+  gate_f32x16 acc;
 #pragma unroll
-      for (int k = 0; k < kRegK; ++k)
-        if (k < K) topk_w[static_cast<size_t>(row) * K + k] = renormalize ? bw[k] / wsum : bw[k];
-    }
-  } else {
-    for (int k = 0; k < K; ++k) {
-      float best;
-      round(k, best);
-      if (live && t == 0) topk_w[static_cast<size_t>(row) * K + k] = best;
-    }
-    if (renormalize && live && t == 0) {
-      for (int k = 0; k < K; ++k) {
-        const size_t o = static_cast<size_t>(row) * K + k;
-        topk_w[o] = topk_w[o] / wsum;
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  const int nu = H / 64;
+  constexpr int AHEAD = kGateRing - 1;  // units in flight
+#pragma unroll
+  for (int u = 0; u < AHEAD; ++u)
+    if (u < nu) issue(u);
+  for (int u = 0; u < nu; ++u) {
+    // unit u has landed (only the AHEAD-1 younger units may be outstanding; near the end
+    // fewer are, and waiting for all of them is as good); everybody has left unit u-1
+    if (u + AHEAD - 1 < nu) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((AHEAD - 1) * kDma) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    asm volatile("s_barrier" ::: "memory");
+    if (u + AHEAD < nu) issue(u + AHEAD);
+    if (worker && wave < NF) {
+      const char* st = smem + (u % kGateRing) * kUnitBytes;
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const uint4 xf = *reinterpret_cast<const uint4*>(st + kWBytes + rd_k[kk]);
+        const uint4 wf = *reinterpret_cast<const uint4*>(st + wave * 32 * kGateRowBytes + rd_k[kk]);
+        acc = gate_mma<El>(wf, xf, acc);
       }
     }
   }
+  __syncthreads();  // the ring is free: it now holds the logits, [token][expert] fp32
+  float* lg = reinterpret_cast<float*>(smem);
+  if (worker && wave < NF) {
+    // acc[r]: expert 32 wave + 8 (r / 4) + 4 lhi + r % 4, token l32; one rounding to the activation dtype
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      lg[l32 * E + wave * 32 + 8 * (r / 4) + 4 * lhi + (r % 4)] = El::ld(El::st(acc[r]));
+  }
+  __syncthreads();
+  if (logits_out) {
+    for (int i = threadIdx.x; i < kGateTokens * E; i += kWave * kGateWaves) {
+      const int row = t0 + i / E;
+      if (row < T) logits_out[static_cast<size_t>(row) * E + i % E] = lg[i];
+    }
+  }
+  // routing, rows in the stand-alone kernel's lane layout
+  constexpr int EPL = G::kEpl, VECS = G::kVecs, VPT = G::kVpt, TPR = G::kTpr, RPW = G::kRowsPerWave;
+  const int t = lane % TPR;
+  for (int r0 = wave * RPW; r0 < kGateTokens; r0 += kGateWaves * RPW) {
+    const int lrow = r0 + lane / TPR;
+    const int row = t0 + lrow;
+    float v[VPT];
+#pragma unroll
+    for (int j = 0; j < VECS; ++j)
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) v[j * EPL + i] = lg[lrow * E + j * EPL * TPR + t * EPL + i];
+    route_row<E>(v, t, row, row < T, topk_w, topk_ids, tok_exp_idx, T, K, renormalize);
+  }
+}
+
+template <typename El, int E>
+void launch_gate(const void* x, const void* wg, float* logits_out, float* w, int32_t* ids,
+                 int32_t* tei, int T, int H, int K, int renorm, hipStream_t s) {
+  using S = typename El::S;
+  const int blocks = (T + kGateTokens - 1) / kGateTokens;
+  // few workgroups (decode): one per CU with a deep ring, 140 KB at E = 128; many: two per CU, 80 KB
+  if (blocks <= 256) {
+    constexpr int lds = 7 * (E + kGateTokens) * kGateRowBytes;
+    auto kern = gate_topk_softmax_kernel<El, E, 7>;
+    static bool attr_set = false;  // dynamic LDS above 64 KB must be opted into
+    if (!attr_set) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(kWave * kGateWaves), lds, s,
+                       static_cast<const S*>(x), static_cast<const S*>(wg), logits_out, w, ids, tei, T, H, K, renorm);
+  } else {
+    constexpr int lds = 4 * (E + kGateTokens) * kGateRowBytes;
+    auto kern = gate_topk_softmax_kernel<El, E, 4>;
+    static bool attr_set = false;
+    if (!attr_set) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(kWave * kGateWaves), lds, s,
+                       static_cast<const S*>(x), static_cast<const S*>(wg), logits_out, w, ids, tei, T, H, K, renorm);
+  }
+}
+
+template <typename El>
+int launch_gate_e(const void* x, const void* wg, float* logits_out, float* w, int32_t* ids,
+                  int32_t* tei, int T, int H, int E, int K, int renorm, hipStream_t s) {
+  switch (E) {
+    case 32: launch_gate<El, 32>(x, wg, logits_out, w, ids, tei, T, H, K, renorm, s); break;
+    case 64: launch_gate<El, 64>(x, wg, logits_out, w, ids, tei, T, H, K, renorm, s); break;
+    case 128: launch_gate<El, 128>(x, wg, logits_out, w, ids, tei, T, H, K, renorm, s); break;
+    default: return moe_fail(MOE_ERR_UNSUPPORTED, "gate_topk_softmax: num_experts %d (32, 64 or 128)", E);
+  }
+  return moe_check_launch("gate_topk_softmax");
 }
 
 // One wavefront per row; lane l holds columns l, l+64, ... (up to 16 of them).
@@ -250,4 +508,29 @@ MOE_EXPORT int moe_topk_softmax(const float* gating_output, float* topk_weights,
     }
   }
   return moe_check_launch("topk_softmax");
+}
+
+MOE_EXPORT int moe_gate_topk_softmax(const void* x, const void* gate_weight, int dtype,
+                                     float* logits_out, float* topk_weights, int32_t* topk_ids,
+                                     int32_t* token_expert_indices, int T, int H, int E, int K,
+                                     int renormalize, void* stream) {
+  if (T < 0 || H < 1 || E < 1 || K < 1) return moe_fail(MOE_ERR_ARG, "gate_topk_softmax: bad sizes T=%d H=%d E=%d K=%d", T, H, E, K);
+  if (K > E) return moe_fail(MOE_ERR_ARG, "gate_topk_softmax: topk %d exceeds num_experts %d", K, E);
+  if (static_cast<int64_t>(T) * K > INT32_MAX)
+    return moe_fail(MOE_ERR_ARG, "gate_topk_softmax: T*K overflows int32 token_expert_indices");
+  if (H % 64 != 0)
+    return moe_fail(MOE_ERR_UNSUPPORTED, "gate_topk_softmax: hidden size %d is not a multiple of 64", H);
+  if (static_cast<int64_t>(T) * H * 2 >= (1LL << 32))
+    return moe_fail(MOE_ERR_UNSUPPORTED, "gate_topk_softmax: x larger than 4 GiB (32-bit row offsets)");
+  if (T == 0) return MOE_OK;
+  if (!x || !gate_weight || !topk_weights || !topk_ids || !token_expert_indices)
+    return moe_fail(MOE_ERR_ARG, "gate_topk_softmax: null pointer");
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gate_weight)) & 15u)
+    return moe_fail(MOE_ERR_ARG, "gate_topk_softmax: x and the gate weight must be 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case MOE_BF16: return launch_gate_e<ElemBF16>(x, gate_weight, logits_out, topk_weights, topk_ids, token_expert_indices, T, H, E, K, renormalize, s);
+    case MOE_F16: return launch_gate_e<ElemF16>(x, gate_weight, logits_out, topk_weights, topk_ids, token_expert_indices, T, H, E, K, renormalize, s);
+    default: return moe_fail(MOE_ERR_UNSUPPORTED, "gate_topk_softmax: dtype code %d (bf16 or fp16)", dtype);
+  }
 }

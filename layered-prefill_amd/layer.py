@@ -15,7 +15,7 @@ from typing import Callable, Optional
 import torch
 import torch.distributed as dist
 
-from .fused_moe import fused_experts, fused_topk
+from .fused_moe import fused_experts, fused_gate_topk, fused_topk
 
 
 @dataclass
@@ -370,3 +370,38 @@ class FusedMoE(torch.nn.Module):
                 f"intermediate_size_per_partition={self.intermediate_size_per_partition}, "
                 f"tp_size={self.tp_size}, renormalize={self.renormalize}, "
                 f"scoring_func='{self.scoring_func}', activation='{self.activation}'")
+
+
+class SparseMoeBlock(torch.nn.Module):
+    """Router gate + experts, the shape of the reference's
+    ``Qwen3MoeSparseMoeBlock`` (nanovllm/models/qwen3_moe.py:70-118): a bias-free
+    gate ``[num_experts, hidden_size]`` (its ``ReplicatedLinear``) and a
+    ``FusedMoE``.  ``forward(hidden_states)`` routes with the fused gate + top-k
+    kernel when the shape allows and hands the experts the routing through
+    ``custom_routing_function``-free plumbing: the result equals
+    ``experts(x, gate(x))``.  TP=1 (the reference's all-reduce at :113-116 is
+    outside this build)."""
+
+    def __init__(self, num_experts: int, top_k: int, hidden_size: int, intermediate_size: int,
+                 params_dtype: Optional[torch.dtype] = None, renormalize: bool = True,
+                 activation: str = "silu", has_bias: bool = False,
+                 quantization: Optional[str] = None):
+        super().__init__()
+        self.experts = FusedMoE(num_experts=num_experts, top_k=top_k, hidden_size=hidden_size,
+                                intermediate_size=intermediate_size, params_dtype=params_dtype,
+                                reduce_results=False, renormalize=renormalize,
+                                activation=activation, has_bias=has_bias, quantization=quantization)
+        self.gate_weight = torch.nn.Parameter(
+            torch.empty(num_experts, hidden_size, dtype=self.experts.params_dtype), requires_grad=False)
+
+    def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        orig_shape = hidden_states.shape
+        x = hidden_states.view(-1, orig_shape[-1])
+        ex = self.experts
+        topk_weights, topk_ids, _ = fused_gate_topk(x, self.gate_weight, ex.top_k, ex.renormalize)
+        out = ex.quant_method.apply(
+            layer=ex, x=x, router_logits=None, top_k=ex.top_k, renormalize=ex.renormalize,
+            activation=ex.activation, apply_router_weight_on_input=ex.apply_router_weight_on_input,
+            global_num_experts=ex.global_num_experts, expert_map=ex.expert_map,
+            custom_routing_function=lambda **_: (topk_weights, topk_ids))
+        return out.view(orig_shape)

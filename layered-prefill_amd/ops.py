@@ -4,6 +4,8 @@ style, nothing returned, work enqueued on torch's current stream.
 """
 from __future__ import annotations
 
+from typing import Optional
+
 import torch
 
 from . import _lib
@@ -51,6 +53,53 @@ def topk_softmax(topk_weights: torch.Tensor, topk_indices: torch.Tensor,
         check(lib().moe_topk_softmax(gating_output.data_ptr(), topk_weights.data_ptr(),
                                      topk_indices.data_ptr(), token_expert_indices.data_ptr(),
                                      T, E, K, int(renormalize), stream_ptr(gating_output.device)))
+
+
+def gate_topk_softmax_supported(hidden_states: torch.Tensor, gate_weight: torch.Tensor) -> bool:
+    """Shapes and dtypes the fused gate + routing kernel takes."""
+    return (hidden_states.dtype in (torch.bfloat16, torch.float16)
+            and gate_weight.dtype == hidden_states.dtype
+            and gate_weight.size(0) in (32, 64, 128) and hidden_states.size(-1) % 64 == 0
+            and hidden_states.is_contiguous() and gate_weight.is_contiguous())
+
+
+def gate_topk_softmax(topk_weights: torch.Tensor, topk_indices: torch.Tensor,
+                      token_expert_indices: torch.Tensor, hidden_states: torch.Tensor,
+                      gate_weight: torch.Tensor, renormalize: bool = False,
+                      logits_out: Optional[torch.Tensor] = None) -> None:
+    """Router gate (``x @ gate_weight.T`` in the activation dtype,
+    nanovllm/models/qwen3_moe.py:93-104,113) and ``topk_softmax`` in one launch.
+    No such op in the reference; out-parameter style as ``topk_softmax``."""
+    require_gpu_tensor(hidden_states, "hidden_states")
+    require_gpu_tensor(gate_weight, "gate_weight")
+    if hidden_states.dtype not in _lib.DTYPE_CODE or gate_weight.dtype != hidden_states.dtype:
+        raise RuntimeError(f"gate_topk_softmax: dtypes {hidden_states.dtype} / {gate_weight.dtype}")
+    if topk_weights.dtype != torch.float32:
+        raise RuntimeError(f"expected scalar type Float but found {topk_weights.dtype}")
+    if topk_indices.dtype != torch.int32 or token_expert_indices.dtype != torch.int32:
+        raise RuntimeError("expected scalar type Int for topk_indices / token_expert_indices")
+    for name, t in (("topk_weights", topk_weights), ("topk_indices", topk_indices),
+                    ("token_expert_indices", token_expert_indices),
+                    ("hidden_states", hidden_states), ("gate_weight", gate_weight)):
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous")
+    T, H = hidden_states.shape
+    E = gate_weight.size(0)
+    K = topk_weights.size(-1)
+    if gate_weight.size(1) != H:
+        raise RuntimeError("gate_topk_softmax: gate_weight must be [num_experts, hidden_size]")
+    if topk_weights.numel() != T * K or topk_indices.numel() != T * K \
+            or token_expert_indices.numel() != T * K:
+        raise RuntimeError("gate_topk_softmax: output tensors must hold num_tokens * topk elements")
+    if logits_out is not None and (logits_out.dtype != torch.float32 or logits_out.numel() != T * E
+                                   or not logits_out.is_contiguous()):
+        raise RuntimeError("gate_topk_softmax: logits_out must be contiguous fp32 [num_tokens, num_experts]")
+    with torch.cuda.device(hidden_states.device):
+        check(lib().moe_gate_topk_softmax(
+            hidden_states.data_ptr(), gate_weight.data_ptr(), _lib.DTYPE_CODE[hidden_states.dtype],
+            logits_out.data_ptr() if logits_out is not None else None, topk_weights.data_ptr(),
+            topk_indices.data_ptr(), token_expert_indices.data_ptr(), T, H, E, K,
+            int(renormalize), stream_ptr(hidden_states.device)))
 
 
 def moe_align_block_size(topk_ids: torch.Tensor, num_experts: int, block_size: int,

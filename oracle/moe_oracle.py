@@ -349,3 +349,20 @@ def fused_experts_fp8_ref(hidden_states: torch.Tensor, w1_q: torch.Tensor, w1_sc
         c2d = dequant_e4m3(cq) * cs[:, None]
         out_k[tok, slot] = _round((c2d @ W2.t()) * tw[tok, slot, None], dt)
     return _round(out_k.sum(dim=1), dt)
+
+
+def gate_logits(hidden_states: torch.Tensor, gate_weight: torch.Tensor) -> torch.Tensor:
+    """Router logits as the reference's gate produces them: a bias-free linear in
+    the activation dtype (nanovllm/models/qwen3_moe.py:93-104,113;
+    nanovllm/layers/linear.py:53-60), i.e. the fp32 product rounded once to that
+    dtype; returned upcast to fp32 as ``fused_topk`` feeds them to the softmax
+    (nanovllm/layers/for_moe/fused_moe.py:409-415).  Pinned by the closed form
+    against ``torch.nn.functional.linear`` in float64 (tests/test_oracle.py)."""
+    acc = hidden_states.float() @ gate_weight.float().t()
+    return acc.to(hidden_states.dtype).float()
+
+
+def gate_topk_softmax(hidden_states: torch.Tensor, gate_weight: torch.Tensor, topk: int,
+                      renormalize: bool = False):
+    """``gate_logits`` followed by ``topk_softmax``."""
+    return topk_softmax(gate_logits(hidden_states, gate_weight), topk, renormalize=renormalize)

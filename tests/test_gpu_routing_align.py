@@ -155,3 +155,67 @@ def test_ops_level_align_signature(moe, oracle, dev):
     assert torch.equal(s.cpu(), os_) and torch.equal(e.cpu(), oe) and n.item() == on.item()
     with pytest.raises(RuntimeError, match="holds"):
         moe.ops.moe_align_block_size(ids, 16, 32, s[:100].contiguous(), e, n)
+
+
+# ------------------------------------------------------------------ fused router gate
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,E,K", [(256, 2048, 128, 8), (700, 512, 64, 4), (33, 256, 32, 2),
+                                     (1, 256, 128, 8), (8448, 2048, 128, 8)])
+def test_gate_topk_softmax_against_oracle(moe, oracle, dev, dtype, T, H, E, K):
+    """Gate GEMM + routing in one kernel.  The logits it routes on (returned
+    through logits_out) must be the oracle's logits up to one rounding step of
+    the activation dtype (the fp32 sum runs in another order), and the routing
+    must be bit-exact for those logits."""
+    print(f"gate_topk_softmax {dtype} T={T} H={H} E={E} K={K}", flush=True)
+    g = torch.Generator().manual_seed(T + H + E)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    wg = (torch.randn(E, H, generator=g) * 0.05).to(dtype)
+    for renorm in (False, True):
+        w = torch.full((T, K), -7.0, dtype=torch.float32, device=dev)
+        ids = torch.full((T, K), -7, dtype=torch.int32, device=dev)
+        tei = torch.full((T, K), -7, dtype=torch.int32, device=dev)
+        logits = torch.full((T, E), float("nan"), dtype=torch.float32, device=dev)
+        moe.ops.gate_topk_softmax(w, ids, tei, x.to(dev), wg.to(dev), renormalize=renorm,
+                                  logits_out=logits)
+        torch.cuda.synchronize()
+        got = logits.cpu()
+        want = oracle.gate_logits(x, wg)
+        # one rounding step of the dtype, plus the fp32 summation-order noise of an
+        # H-term dot product where the terms cancel to a small logit
+        ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+        assert ((got - want).abs() <= 2 * ulp * want.abs() + 3e-5).all()
+        assert (got != want).float().mean() < 0.05          # a different rounding is the exception
+        assert torch.equal(got, got.to(dtype).float())       # values of the activation dtype
+        ow, oids, otei = oracle.topk_softmax(got, K, renormalize=renorm)
+        assert torch.equal(ids.cpu(), oids) and torch.equal(tei.cpu(), otei)
+        assert torch.equal(w.cpu().view(torch.int32), ow.view(torch.int32))
+
+
+def test_fused_gate_topk_falls_back_and_block_matches_two_step(moe, oracle, dev, monkeypatch):
+    g = torch.Generator().manual_seed(11)
+    # unsupported expert count: the gate runs as a plain linear, then fused_topk
+    x = torch.randn(50, 256, generator=g).bfloat16().to(dev)
+    wg = (torch.randn(48, 256, generator=g) * 0.05).bfloat16().to(dev)
+    w, ids, _ = moe.fused_gate_topk(x, wg, 4, True)
+    w2, ids2, _ = moe.fused_topk(x, torch.nn.functional.linear(x, wg), 4, True)
+    assert torch.equal(ids, ids2) and torch.equal(w, w2)
+    with pytest.raises(RuntimeError, match="num_experts 48"):
+        moe.ops.gate_topk_softmax(w, ids, ids.clone(), x, wg)
+    # the block: gate + experts, against the same experts fed with its own routing
+    monkeypatch.setattr(moe.fused_moe, "FUSED_GATE_MIN_TOKENS", 1)   # take the fused kernel at this size
+    E, H, I, T, K = 32, 256, 128, 200, 4
+    blk = moe.SparseMoeBlock(E, K, H, I, params_dtype=torch.bfloat16).to(dev)
+    blk.gate_weight.data.copy_((torch.randn(E, H, generator=g) * 0.05).bfloat16())
+    blk.experts.w13_weight.data.copy_((torch.randn(E, 2 * I, H, generator=g) * 0.05).bfloat16())
+    blk.experts.w2_weight.data.copy_((torch.randn(E, H, I, generator=g) * 0.05).bfloat16())
+    xs = torch.randn(4, 50, H, generator=g).bfloat16().to(dev)   # leading dims are flattened
+    out = blk(xs.clone())
+    assert out.shape == xs.shape
+    flat = xs.view(-1, H)
+    tw, tids, _ = moe.fused_gate_topk(flat, blk.gate_weight.data, K, True)
+    ref = moe.fused_experts(flat, blk.experts.w13_weight.data, blk.experts.w2_weight.data, None, None,
+                            tw, tids)
+    assert torch.equal(out.view(-1, H), ref)
+    full = oracle.fused_experts_ref(flat.cpu(), blk.experts.w13_weight.data.cpu(),
+                                    blk.experts.w2_weight.data.cpu(), tw.cpu(), tids.cpu())
+    assert (out.view(-1, H).float().cpu() - full).abs().max() < 1e-2 + 2e-2 * full.abs().max()

@@ -330,3 +330,21 @@ def test_mirrored_rounding_stays_close_to_fp32(oracle):
     a = oracle.fused_experts_ref(x, w13, w2, w, ids)
     b = oracle.fused_experts_ref(x, w13, w2, w, ids, mirror_rounding=True)
     assert torch.allclose(a, b, rtol=2e-2, atol=1e-2)
+
+
+def test_gate_logits_are_the_float64_linear_rounded_once(oracle):
+    """The router gate is a bias-free linear whose output has the activation
+    dtype: against float64 `linear` rounded to that dtype only a double rounding
+    can differ (fp32 sum first), and then by one step."""
+    g = torch.Generator().manual_seed(3)
+    for dtype, ulp in ((torch.bfloat16, 2.0 ** -7), (torch.float16, 2.0 ** -10)):  # spacing / value, at most
+        x = torch.randn(64, 512, generator=g).to(dtype)
+        w = (torch.randn(128, 512, generator=g) * 0.05).to(dtype)
+        got = oracle.gate_logits(x, w)
+        want = torch.nn.functional.linear(x.double(), w.double()).to(dtype).float()
+        assert got.dtype == torch.float32 and got.shape == (64, 128)
+        assert ((got - want).abs() <= ulp * want.abs() + 1e-7).all()
+        assert (got != want).float().mean() < 0.01
+        tw, ids, _ = oracle.gate_topk_softmax(x, w, 4, renormalize=True)
+        tw2, ids2, _ = oracle.topk_softmax(got, 4, renormalize=True)
+        assert torch.equal(ids, ids2) and torch.equal(tw, tw2)
