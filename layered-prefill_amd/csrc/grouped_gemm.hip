@@ -645,7 +645,7 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
 // Epilogue phase 1: round this wavefront's accumulators to the activation dtype
 // (after the optional bias and routed weight) and park them in its LDS window
 // as [token row][weight row].
-template <typename El, int FMC, bool GATED, bool SCALED>
+template <typename El, int FMC, bool GATED, bool SCALED, bool BIAS>
 __device__ __forceinline__ void big_park(const GemmParams& p, int e, int n0, int wn, int lhi, int l32,
                                          const float* s_rw, const float* s_as, char* epi,
                                          const f32x16 (&acc)[4][4]) {
@@ -688,14 +688,13 @@ __device__ __forceinline__ void big_park(const GemmParams& p, int e, int n0, int
 #pragma unroll
           for (int i = 0; i < 4; ++i) v[i] *= as * ws[fn * 16 + 4 * g + i];
         }
-        if (bias) {
+        if constexpr (BIAS) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) v[i] += El::ld(bias[e * p.bias_stride_e + wrow_of(fn, g, i)]);
         }
-        if (p.mul_weight) {
+        // rw is exactly 1 when the routed weight is not applied in this pass
 #pragma unroll
-          for (int i = 0; i < 4; ++i) v[i] *= rw;
-        }
+        for (int i = 0; i < 4; ++i) v[i] *= rw;
         *reinterpret_cast<uint2*>(row + (fn * 32 + 8 * g + 4 * lhi) * 2) =
             uint2{pack2<El>(v[0], v[1]), pack2<El>(v[2], v[3])};
       }
@@ -750,6 +749,34 @@ __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, i
   const int c8 = (lane % LPR) * 8;
   const int ncol = n0 + wn * COLS + c8;
   const bool vec_ok = ncol + 7 < p.N && (p.ldc & 7) == 0;
+  // Whole wavefront inside the matrix: no per-lane edge handling.  Real slots come
+  // first in a block, so row r is live exactly when r < rows.
+  if (n0 + wn * COLS + COLS <= p.N && (p.ldc & 7) == 0) {
+    const int lrow = lane / LPR;
+    char* const cbase = static_cast<char*>(p.c) + static_cast<int64_t>(ncol) * 2;
+    const int64_t ldc_bytes = static_cast<int64_t>(p.ldc) * 2;
+    const char* src = epi + lrow * kEpiRowBytes + c8 * 2;
+    for (int r0 = 0; r0 < rows; r0 += RPS * UNR) {
+      int crow[UNR];
+      uint4 gq[UNR], uq[UNR];
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
+        const int r = r0 + u * RPS + lrow;  // < 128: rows <= 128 and 128 is a multiple of RPS * UNR
+        crow[u] = p.a_by_slot ? s_tok[r] : slot0 + r;
+        gq[u] = *reinterpret_cast<const uint4*>(src + (r0 + u * RPS) * kEpiRowBytes);
+        if constexpr (GATED) uq[u] = *reinterpret_cast<const uint4*>(src + (r0 + u * RPS) * kEpiRowBytes + 128);
+      }
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
+        uint4 out = gq[u];
+        if constexpr (GATED)
+          out = uint4{gated_pair<El, ACT>(p, gq[u].x, uq[u].x), gated_pair<El, ACT>(p, gq[u].y, uq[u].y),
+                      gated_pair<El, ACT>(p, gq[u].z, uq[u].z), gated_pair<El, ACT>(p, gq[u].w, uq[u].w)};
+        if (r0 + u * RPS + lrow < rows) *reinterpret_cast<uint4*>(cbase + crow[u] * ldc_bytes) = out;
+      }
+    }
+    return;
+  }
   for (int r0 = 0; r0 < rows; r0 += RPS * UNR) {
     int tok[UNR];
     uint4 gq[UNR], uq[UNR];
@@ -796,15 +823,24 @@ __device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, c
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[fn][fm][r] = 0.f;
   big_mainloop<Mma, FMC>(c, smem, nk, acc);
+#ifdef MOE_TRACE
+  if (threadIdx.x == 0 && blockIdx.x < 4096) moe_dbg[blockIdx.x * 8 + 7] = MOE_TRACE_NOW();
+#endif
   bare_barrier();  // every wavefront is done reading the ring before it is reused
   s_tok_all[threadIdx.x] = my_tok;
   s_rw_all[threadIdx.x] = my_rw;  // requested before the main loop, needed only now
   s_rw_all[kBigBM + threadIdx.x] = my_as;
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   bare_barrier();
-  if constexpr (FMC > 0)
-    big_park<El, FMC, GATED, Mma::kEs == 1>(p, e, n0, wn, lane >> 5, lane & 31, s_rw_all + wm * 128,
-                                            s_rw_all + kBigBM + wm * 128, epi, acc);
+  if constexpr (FMC > 0) {
+    // one straight-line body per case: a test per element costs more than the element
+    if (p.bias)
+      big_park<El, FMC, GATED, Mma::kEs == 1, true>(p, e, n0, wn, lane >> 5, lane & 31, s_rw_all + wm * 128,
+                                                    s_rw_all + kBigBM + wm * 128, epi, acc);
+    else
+      big_park<El, FMC, GATED, Mma::kEs == 1, false>(p, e, n0, wn, lane >> 5, lane & 31, s_rw_all + wm * 128,
+                                                     s_rw_all + kBigBM + wm * 128, epi, acc);
+  }
 }
 
 template <typename Mma, bool GATED>
@@ -834,7 +870,7 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   [[maybe_unused]] const unsigned long long t_start = MOE_TRACE_NOW();
   [[maybe_unused]] const unsigned long long c_start = __builtin_readcyclecounter();
   // the two loads below do not depend on each other: one memory latency, not two
-  const int e = p.expert_ids[(mb * kBigBM) / p.align_bs];
+  const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[(mb * kBigBM) / p.align_bs]);
   const int64_t my_slot = static_cast<int64_t>(mb) * kBigBM + tid;
   const int my_tok = p.sorted_ids[my_slot < p.sorted_cap ? my_slot : p.sorted_cap - 1];
   const int n0 = nt * (GATED ? kBigBNW / 2 : kBigBNW);
