@@ -482,6 +482,7 @@ struct IntTag { static constexpr int value = V; };
 
 // Main loop for a wavefront that has FMC live token fragments (0..4).
 // Unit j of the stream  A(0) W(0) A(1) W(1) ...  lives in ring slot j % 5.
+// The caller has requested W(0) and W(1) (when nk > 1) before anything else.
 // One K tile (128 bytes per row) is STEPS MFMA steps of CH 16-byte chunks per
 // lane and operand: four steps of one chunk for the 16-bit dtypes, two steps
 // of two chunks for e4m3.  Two register sets of fragments (P, Q) alternate,
@@ -506,10 +507,6 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
   auto issue_a = [&](int kt, int slot) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) dma_a(kt, slot, i);
-  };
-  auto issue_w = [&](int kt, int slot) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) dma_w(kt, slot, i);
   };
   constexpr int XF = FMC > 0 ? FMC : 1;
   auto read_frags = [&](int sa, int sw, int kk, uint4 (&wf)[4][CH], uint4 (&xf)[XF][CH]) {
@@ -572,13 +569,13 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
   using Tag4 = IntTag<4>;
   using TagPer = IntTag<PER>;
 
-  // fill the ring: A(0) W(0) A(1) W(1) A(2), then wait for tile 0 only
+  // fill the ring: W(0) and W(1) were requested by the caller as soon as it knew the
+  // expert; A(0) A(1) A(2) follow here.  Then wait for tile 0 only.
   issue_a(0, 0);
-  issue_w(0, 1);
-  if (1 < nk) { issue_a(1, 2); issue_w(1, 3); }
+  if (1 < nk) issue_a(1, 2);
   if (2 < nk) issue_a(2, 4);
-  if (2 < nk) wait_vmcnt<3 * kBigDmaPerUnit>();
-  else if (1 < nk) wait_vmcnt<2 * kBigDmaPerUnit>();
+  if (2 < nk) wait_vmcnt<2 * kBigDmaPerUnit>();
+  else if (1 < nk) wait_vmcnt<kBigDmaPerUnit>();
   else wait_vmcnt<0>();
   bare_barrier();
   int sa = 0, sw = 1;  // slots of the tile being multiplied
@@ -881,32 +878,16 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   int* s_cnt = reinterpret_cast<int*>(smem + kBigLdsBytes + kBigSideBytes);
   const int wave_cnt = __popcll(__ballot(my_tok < p.numel));
   if (lane == 0) s_cnt[wave] = wave_cnt;
-  __syncthreads();
-  const int nvalid = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
-  if (nvalid == 0) return;
-  float my_rw = 1.f, my_as = 1.f;
-  if (p.mul_weight) my_rw = my_tok < p.numel ? p.topk_w[my_tok] : 0.f;
-  if (p.a_scale && my_tok < p.numel) my_as = p.a_scale[p.a_by_slot ? my_slot : my_tok / p.top_k];
   constexpr int ES = Mma::kEs, CH = Mma::kBigChunks;
-
+  const int nk = p.Kd / (kBigRowBytes / ES);
   BigCtx c;
   const int ld_row = tid >> 3;                        // row inside a 32-row load group
   const int ld_chunk = (tid & 7) ^ ((tid >> 4) & 7);  // logical chunk this lane fetches
   c.a_base = static_cast<const char*>(p.a);
   c.w_base = static_cast<const char*>(p.w) + static_cast<int64_t>(e) * p.w_stride_e * ES;
-  const int a_groups = (nvalid + 31) >> 5;  // 32-row token groups that hold real slots
+  c.dma_lds = __builtin_amdgcn_readfirstlane(lds_offset_of(smem) + wave * 1024);
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    // groups made of padding only re-request group 0 (an L1 hit) so that every
-    // token unit is exactly eight loads and the vmcnt bookkeeping stays fixed
-    const int gi = i < a_groups ? i : 0;
-    const int slot = mb * kBigBM + ld_row + 32 * gi;
-    int64_t src = slot;
-    if (!p.a_by_slot) {
-      const int tok = s_tok[ld_row + 32 * gi];
-      src = tok < p.numel ? tok / p.top_k : 0;
-    }
-    c.a_off[i] = static_cast<uint32_t>(src * p.lda * ES + ld_chunk * 16);
     const int rr = ld_row + 32 * i;
     int64_t wrow;
     if constexpr (GATED) {
@@ -920,7 +901,39 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
     }
     c.w_off[i] = static_cast<uint32_t>(wrow * p.w_stride_n * ES + ld_chunk * 16);
   }
-  c.dma_lds = __builtin_amdgcn_readfirstlane(lds_offset_of(smem) + wave * 1024);
+  // The weights of the first two K tiles are on their way (ring slots 1 and 3) while
+  // the slot ids are still being looked at: they are the cold half of the fill.
+  // Neither slot overlaps the side arrays above.
+#pragma unroll
+  for (int i = 0; i < 8; ++i) lds_dma16(c.w_base, c.w_off[i], c.dma_lds + kBigUnitBytes + i * 4096);
+  if (1 < nk) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      lds_dma16(c.w_base + kBigRowBytes, c.w_off[i], c.dma_lds + 3 * kBigUnitBytes + i * 4096);
+  }
+  __syncthreads();
+  const int nvalid = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
+  if (nvalid == 0) {
+    wait_vmcnt<0>();  // nothing may still be landing in LDS when the workgroup ends
+    return;
+  }
+  float my_rw = 1.f, my_as = 1.f;
+  if (p.mul_weight) my_rw = my_tok < p.numel ? p.topk_w[my_tok] : 0.f;
+  if (p.a_scale && my_tok < p.numel) my_as = p.a_scale[p.a_by_slot ? my_slot : my_tok / p.top_k];
+  const int a_groups = (nvalid + 31) >> 5;  // 32-row token groups that hold real slots
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    // groups made of padding only re-request group 0 (an L1 hit) so that every
+    // token unit is exactly eight loads and the vmcnt bookkeeping stays fixed
+    const int gi = i < a_groups ? i : 0;
+    const int slot = mb * kBigBM + ld_row + 32 * gi;
+    int64_t src = slot;
+    if (!p.a_by_slot) {
+      const int tok = s_tok[ld_row + 32 * gi];
+      src = tok < p.numel ? tok / p.top_k : 0;
+    }
+    c.a_off[i] = static_cast<uint32_t>(src * p.lda * ES + ld_chunk * 16);
+  }
   // chunk ch of MFMA step kk: lane half lhi owns the K elements of chunks CH * (2 kk + lhi) .. + CH - 1
 #pragma unroll
   for (int q = 0; q < 4; ++q)
@@ -935,7 +948,6 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
       r = wn * 128 + fn * 32;
     c.w_row[fn] = r * kBigRowBytes;
   }
-  const int nk = p.Kd / (kBigRowBytes / ES);
   const int slot0 = mb * kBigBM + wm * 128;
   char* epi = smem + wave * kEpiWaveBytes;
   [[maybe_unused]] const unsigned long long t_pro = MOE_TRACE_NOW();
