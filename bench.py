@@ -147,10 +147,12 @@ def time_graph_replays(layer: Layer, steps: int, warmup: int):
 
 
 def time_router_gate(moe, layer: Layer, steps: int):
-    """Router gate ahead of the measured path (SURVEY 8f-2 of the scope table is
-    the fused form): gate linear + fused_topk as two steps, as the reference runs
-    them (nanovllm/models/qwen3_moe.py:93-104,113), against the one-kernel
-    fused_gate_topk.  Microseconds per call, events around `steps` calls."""
+    """The two steps ahead of the measured path: the residual add + RMSNorm that
+    produces the block's input (csrc/layernorm_kernels.cu:77-108 of the reference;
+    four tensors of T*H elements move once each) and the router gate, as gate linear
+    + fused_topk the way the reference runs them (nanovllm/models/qwen3_moe.py:93-104,113)
+    against the one-kernel fused_gate_topk.  Microseconds per call, events around
+    `steps` calls."""
     s = layer.shape
     g = torch.Generator().manual_seed(99)
     wg = (torch.randn(s.experts, s.hidden, generator=g) * 0.02).to(layer.x.dtype).to(layer.dev)
@@ -161,8 +163,15 @@ def time_router_gate(moe, layer: Layer, steps: int):
     def fused():
         return moe.fused_gate_topk(layer.x, wg, s.top_k, True)
 
+    res = torch.randn_like(layer.x)
+    normed = torch.empty_like(layer.x)
+    wn = torch.ones(s.hidden, dtype=layer.x.dtype, device=layer.dev)
+
+    def norm():
+        moe.ops.add_rms_norm(normed, res, layer.x, wn, 1e-6)
+
     out = {}
-    for name, fn in (("linear_then_topk_us", two_step), ("fused_gate_topk_us", fused)):
+    for name, fn in (("linear_then_topk_us", two_step), ("fused_gate_topk_us", fused), ("add_rms_norm_us", norm)):
         for _ in range(5):
             fn()
         ev = _events(2)
@@ -172,7 +181,60 @@ def time_router_gate(moe, layer: Layer, steps: int):
         ev[1].record()
         torch.cuda.synchronize()
         out[name] = round(ev[0].elapsed_time(ev[1]) * 1e3 / steps, 2)
+    out["add_rms_norm_gbs"] = round(4 * layer.x.numel() * layer.x.element_size() / out["add_rms_norm_us"] * 1e-3, 1)
     return out
+
+
+def trace_mix(moe, layer: Layer, steps: int):
+    """Layer calls as a layered-prefill engine would issue them on the ShareGPT length
+    sample: the schedule (nanovllm/engine/scheduler.py:181-328 restated on the host) over
+    400 requests with Poisson arrivals, a 48-layer model, 16 configured stages, 256
+    sequences and 8192 prompt tokens per group at most.  Call sizes are bucketed (64-token
+    steps up to 512 tokens, 1024-token steps above), the buckets that carry the most tokens
+    are timed with this layer's weights, and the token throughput of the mix is reported."""
+    sch = moe.schedule
+    wl = moe.workloads
+    s = layer.shape
+    num_layers = 48
+    reqs = sch.poisson_requests(sch.load_length_trace(), 400, per_iteration=0.4, seed=0)
+    shapes = sch.simulate(reqs, num_layers=num_layers, configured_stages=16, max_num_seqs=256,
+                          max_num_batched_tokens=8192)
+    sizes = sch.moe_call_sizes(shapes, num_layers)
+    buckets = {}
+    for t, calls in sizes.items():
+        b = -(-t // 64) * 64 if t <= 512 else max(1024, int(round(t / 1024.0)) * 1024)
+        c, tok = buckets.get(b, (0, 0))
+        buckets[b] = (c + calls, tok + calls * t)
+    total_tok = sum(tok for _, tok in buckets.values())
+    total_calls = sum(c for c, _ in buckets.values())
+    picked = sorted(buckets, key=lambda b: -buckets[b][1])[:6]
+    rows, t_ms, t_tok = [], 0.0, 0
+    for b in sorted(picked):
+        x, logits = wl.make_inputs(s, b, 700 + b, layer.x.dtype)
+        x, logits = x.to(layer.dev), logits.to(layer.dev)
+
+        def step():
+            tw, ids, _ = moe.fused_topk(x, logits, s.top_k, True)
+            return moe.fused_experts(x, layer.w13, layer.w2, None, None, tw, ids)
+
+        for _ in range(3):
+            step()
+        ev = _events(2)
+        ev[0].record()
+        for _ in range(steps):
+            step()
+        ev[1].record()
+        torch.cuda.synchronize()
+        ms = ev[0].elapsed_time(ev[1]) / steps
+        calls, tok = buckets[b]
+        rows.append({"tokens": b, "calls_share": round(calls / total_calls, 4),
+                     "tokens_share": round(tok / total_tok, 4), "ms": round(ms, 4)})
+        t_ms += calls * ms
+        t_tok += tok
+    return {"trace": "sharegpt_8k_lengths_first2048.csv", "requests": len(reqs), "iterations": len(shapes),
+            "layers": num_layers, "stages": 16, "buckets": rows,
+            "covered_tokens_share": round(t_tok / total_tok, 4),
+            "layer_tokens_per_s": round(t_tok / (t_ms * 1e-3), 0)}
 
 
 def time_stages(layer: Layer, steps: int):
@@ -277,6 +339,8 @@ def main() -> int:
                          "rocprofv3 counter runs), or off")
     ap.add_argument("--no-fp8", action="store_true", help="skip the e4m3 leg (config 5)")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay of the decode leg")
+    ap.add_argument("--no-trace-mix", action="store_true",
+                    help="skip the layered-prefill call-size mix of the ShareGPT length sample")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 1 GiB device copies, the known-size kernel that "
                          "FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -357,6 +421,8 @@ def main() -> int:
     }
 
     out["router_gate"] = time_router_gate(moe, main_layer, 50)
+    if compute_bound and not a.no_trace_mix:
+        out["trace_mix"] = trace_mix(moe, main_layer, 10)
     if compute_bound and a.chunk_mode != "off":
         out["chunk_amplification"] = chunk_amplification(moe, main_layer, max(2, a.steps // 10), a.chunk_mode)
     if compute_bound and not a.no_fp8:

@@ -93,6 +93,16 @@ int moe_silu_and_mul(void* out, const void* in, int64_t rows, int d, int dtype, 
 int moe_swigluoai_and_mul(void* out, const void* in, int64_t rows, int d, int dtype, float alpha,
                           float limit, void* stream);
 
+/* Replaces `add_rms_norm` and `rms_norm` for 2-D inputs (csrc/layernorm_kernels.cu:205-232
+ * and :151-176, kernels :77-108 and :10-35, bound at csrc/ops.cpp:16-27,103-109): the norm
+ * in front of the MoE block.  residual != NULL: s = x + residual in fp32, residual = T(s),
+ * out = T(T(residual * rsqrt(mean(s^2) + eps)) * weight); residual == NULL: the same with
+ * s = x and nothing stored back.  Strides are element strides of dimension 0; the last
+ * dimension is contiguous.  `out` may be `x`. */
+int moe_add_rms_norm(void* out, int64_t out_stride, void* residual, int64_t residual_stride,
+                     const void* x, int64_t x_stride, const void* weight, int dtype, int64_t T,
+                     int H, float eps, void* stream);
+
 /* Replaces `moe_sum` (nanovllm/layers/for_moe/moe_easy_kernel.py:26-31):
  * out[t,:] = sum_k in[t,k,:], fp32 accumulation, one rounding. */
 int moe_sum(void* out, const void* in, int64_t T, int K, int H, int dtype, void* stream);

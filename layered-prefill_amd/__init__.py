@@ -11,9 +11,9 @@ the Triton grouped GEMM of scale-snu/layered-prefill.
 Everything computes through libmoe_gfx950.so (hand-written HIP); there is no
 CPU or PyTorch fallback.
 """
-from . import _lib, ops, fused_moe, layer, loader, workloads  # noqa: F401
+from . import _lib, ops, fused_moe, layer, loader, schedule, workloads  # noqa: F401
 from .fused_moe import (fused_experts, fused_experts_impl, fused_gate_topk, fused_topk,  # noqa: F401
                         moe_align_block_size, quantize_expert_weights,
                         try_get_optimal_moe_config)
 from .layer import (FusedMoE, FusedMoEParallelConfig, MoEConfig, UnquantizedFusedMoEMethod,  # noqa: F401
-                    Fp8E4M3FusedMoEMethod, SparseMoeBlock)
+                    Fp8E4M3FusedMoEMethod, GptOssMLP, RMSNorm, SparseMoeBlock)

@@ -26,7 +26,7 @@ EXPORTS = (
     "moe_last_error", "moe_abi_version", "moe_topk_softmax", "moe_align_workspace_bytes",
     "moe_align_block_size", "moe_silu_and_mul", "moe_swigluoai_and_mul", "moe_sum",
     "moe_fused_experts_workspace_bytes", "moe_fused_experts", "moe_preferred_block_size",
-    "moe_quant_rows_e4m3", "moe_gate_topk_softmax",
+    "moe_quant_rows_e4m3", "moe_gate_topk_softmax", "moe_add_rms_norm",
 )
 
 
@@ -88,6 +88,8 @@ def _declare(L: ctypes.CDLL) -> None:
     L.moe_preferred_block_size.argtypes = [i32] * 5
     L.moe_quant_rows_e4m3.restype = i32
     L.moe_quant_rows_e4m3.argtypes = [p, i32, i64, i32, p, p, p]
+    L.moe_add_rms_norm.restype = i32
+    L.moe_add_rms_norm.argtypes = [p, i64, p, i64, p, i64, p, i32, i64, i32, f32, p]
 
 
 def lib() -> ctypes.CDLL:

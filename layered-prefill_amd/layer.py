@@ -15,6 +15,7 @@ from typing import Callable, Optional
 import torch
 import torch.distributed as dist
 
+from . import ops
 from .fused_moe import fused_experts, fused_gate_topk, fused_topk
 
 
@@ -405,3 +406,51 @@ class SparseMoeBlock(torch.nn.Module):
             global_num_experts=ex.global_num_experts, expert_map=ex.expert_map,
             custom_routing_function=lambda **_: (topk_weights, topk_ids))
         return out.view(orig_shape)
+
+
+class GptOssMLP(torch.nn.Module):
+    """The gpt-oss form of the block, the shape of the reference's ``GptOssMLP``
+    (nanovllm/models/gpt_oss.py:120-158): a router linear *with* bias and experts
+    with ``w13_bias`` / ``w2_bias`` and the interleaved, clamped ``swigluoai``
+    activation.  ``forward(x)`` = ``experts(x, router(x))``.  The router is a plain
+    library GEMM (its bias keeps it off the fused gate kernel).  TP=1."""
+
+    def __init__(self, num_local_experts: int, num_experts_per_tok: int, hidden_size: int,
+                 intermediate_size: int, params_dtype: Optional[torch.dtype] = torch.bfloat16):
+        super().__init__()
+        self.num_experts = num_local_experts
+        self.top_k = num_experts_per_tok
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.router = torch.nn.Linear(hidden_size, num_local_experts, dtype=params_dtype)
+        self.experts = FusedMoE(num_experts=num_local_experts, top_k=num_experts_per_tok,
+                                hidden_size=hidden_size, intermediate_size=intermediate_size,
+                                params_dtype=params_dtype, reduce_results=False, renormalize=True,
+                                has_bias=True, activation="swigluoai")
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        g = self.router(x)
+        return self.experts(hidden_states=x, router_logits=g)
+
+
+class RMSNorm(torch.nn.Module):
+    """The norm in front of the MoE block, same interface as the reference's
+    ``RMSNorm`` (nanovllm/layers/layernorm.py:7-34): ``forward(x)`` returns the
+    normalised tensor, ``forward(x, residual)`` adds ``x`` into ``residual`` in
+    place first and returns ``(out, residual)``."""
+
+    def __init__(self, hidden_size: int, eps: float = 1e-6) -> None:
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.eps = eps
+        self.weight = torch.nn.Parameter(torch.ones(hidden_size))
+
+    def forward(self, x: torch.Tensor, residual: Optional[torch.Tensor] = None,
+                out: Optional[torch.Tensor] = None):
+        if out is None:
+            out = torch.empty_like(x)
+        if residual is None:
+            ops.rms_norm(out, x, self.weight.data, self.eps)
+            return out
+        ops.add_rms_norm(out, residual, x, self.weight.data, self.eps)
+        return out, residual

@@ -181,6 +181,42 @@ def moe_sum(input: torch.Tensor, output: torch.Tensor) -> None:
                             _lib.DTYPE_CODE[input.dtype], stream_ptr(input.device)))
 
 
+def _norm_call(out, residual, x, weight, eps, name):
+    require_gpu_tensor(x, "x")
+    if x.dim() != 2:
+        raise RuntimeError(f"{name}: only [num_tokens, hidden_size] inputs are supported "
+                           "(the per-head form is used by attention, not by the MoE block)")
+    if x.dtype not in _lib.DTYPE_CODE:
+        raise RuntimeError(f"{name} not implemented for '{x.dtype}'")
+    T, H = x.shape
+    tensors = [("out", out), ("x", x)] + ([("residual", residual)] if residual is not None else [])
+    for nm, t in tensors:
+        if tuple(t.shape) != (T, H) or t.dtype != x.dtype or t.device != x.device:
+            raise RuntimeError(f"{name}: {nm} must be [{T}, {H}] of dtype {x.dtype} on {x.device}")
+        if t.stride(1) != 1:
+            raise RuntimeError(f"{name}: {nm} must be contiguous in its last dimension")
+    if tuple(weight.shape) != (H,) or weight.dtype != x.dtype or not weight.is_contiguous():
+        raise RuntimeError(f"{name}: weight must be a contiguous [{H}] tensor of dtype {x.dtype}")
+    with torch.cuda.device(x.device):
+        check(lib().moe_add_rms_norm(out.data_ptr(), out.stride(0),
+                                     residual.data_ptr() if residual is not None else None,
+                                     residual.stride(0) if residual is not None else 0,
+                                     x.data_ptr(), x.stride(0), weight.data_ptr(),
+                                     _lib.DTYPE_CODE[x.dtype], T, H, float(eps), stream_ptr(x.device)))
+
+
+def rms_norm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float) -> None:
+    """csrc/layernorm_kernels.cu:151-176 (2-D case): out = T(T(x * rsqrt(mean(x^2) + eps)) * weight)."""
+    _norm_call(out, None, x, weight, eps, "rms_norm")
+
+
+def add_rms_norm(out: torch.Tensor, residual: torch.Tensor, x: torch.Tensor, weight: torch.Tensor,
+                 eps: float) -> None:
+    """csrc/layernorm_kernels.cu:205-232 (2-D case): residual += x (rounded to the dtype),
+    out = rms_norm(residual).  Argument order as in nanovllm/layers/custom_ops.py:40-41."""
+    _norm_call(out, residual, x, weight, eps, "add_rms_norm")
+
+
 def quant_rows_e4m3(w: torch.Tensor):
     """[..., cols] -> (e4m3fn codes as uint8 of the same shape, fp32 scales [...]):
     per-row s = amax|w| / 448.  No counterpart in the reference."""

@@ -366,3 +366,24 @@ def gate_topk_softmax(hidden_states: torch.Tensor, gate_weight: torch.Tensor, to
                       renormalize: bool = False):
     """``gate_logits`` followed by ``topk_softmax``."""
     return topk_softmax(gate_logits(hidden_states, gate_weight), topk, renormalize=renormalize)
+
+
+def add_rms_norm(x: torch.Tensor, residual: Optional[torch.Tensor], weight: torch.Tensor,
+                 eps: float):
+    """The norm in front of the MoE block, csrc/layernorm_kernels.cu:77-108
+    (``add_rms_norm_kernel``) and :10-35 (``rms_norm_kernel``) of the reference:
+    s = float(x) + float(residual); residual' = T(s); the variance is the mean of
+    s*s over the row (s before rounding, :91-94); out = T(T(float(residual') * r) *
+    weight) with r = rsqrt(variance + eps) (:97-107).  The mean is taken in float64
+    here and r rounded to fp32 once, so results can differ from an fp32 reduction
+    in the last place of r.  Returns ``(out, residual')`` (``residual'`` is None
+    without a residual).  Pinned by known answers in tests/test_oracle.py."""
+    dt = x.dtype
+    s32 = x.float() if residual is None else x.float() + residual.float()
+    new_res = None if residual is None else s32.to(dt)
+    var = (s32.double() * s32.double()).mean(dim=-1, keepdim=True)
+    r = (1.0 / torch.sqrt(var + float(eps))).float()
+    base = s32 if residual is None else new_res.float()
+    normed = (base * r).to(dt)
+    out = (normed.float() * weight.float()).to(dt)
+    return out, new_res

@@ -361,3 +361,34 @@ def test_random_shapes_all_kernels(moe, oracle, dev, case, monkeypatch):
         out = moe.fused_experts(d(x), d(w13), d(w2), None, None, d(tw), d(ids))
         ref = oracle.fused_experts_ref(x, w13, w2, tw, ids, mirror_rounding=True)
         _close(out, ref, rtol=1.6e-2, atol=2e-3 + 4e-3 * ref.abs().max().item())
+
+
+@pytest.mark.gpu
+def test_gpt_oss_mlp_block(moe, oracle, dev):
+    """nanovllm/models/gpt_oss.py:120-158: router linear with bias, experts with biases and
+    the interleaved swigluoai activation, renormalised top-k.  The routing is checked
+    bit-exactly on the router logits the GPU produced, the output against the fp32 oracle."""
+    E, H, I, T, K = 32, 256, 128, 90, 4
+    g = torch.Generator().manual_seed(17)
+    blk = moe.GptOssMLP(E, K, H, I).to(dev)
+    ex = blk.experts
+    assert ex.activation == "swigluoai" and ex.renormalize and hasattr(ex, "w13_bias")
+    blk.router.weight.data.copy_((torch.randn(E, H, generator=g) * 0.05).bfloat16())
+    blk.router.bias.data.copy_((torch.randn(E, generator=g) * 0.5).bfloat16())
+    ex.w13_weight.data.copy_((torch.randn(E, 2 * I, H, generator=g) * 0.05).bfloat16())
+    ex.w2_weight.data.copy_((torch.randn(E, H, I, generator=g) * 0.05).bfloat16())
+    ex.w13_bias.data.copy_((torch.randn(E, 2 * I, generator=g) * 0.1).bfloat16())
+    ex.w2_bias.data.copy_((torch.randn(E, H, generator=g) * 0.1).bfloat16())
+    x = torch.randn(T, H, generator=g).bfloat16()
+    xd = x.to(dev)
+    logits = blk.router(xd)
+    # the router is a linear in the activation dtype: fp32 sum + bias, one rounding
+    want_logits = torch.nn.functional.linear(x.double(), blk.router.weight.data.cpu().double(),
+                                             blk.router.bias.data.cpu().double())
+    assert ((logits.cpu().double() - want_logits).abs() <= 2.0 ** -7 * want_logits.abs() + 1e-6).all()
+    out = blk(xd.clone())
+    tw, ids, _ = oracle.topk_softmax(logits.float().cpu(), K, renormalize=True)
+    ref = oracle.fused_experts_ref(x, ex.w13_weight.data.cpu(), ex.w2_weight.data.cpu(), tw, ids,
+                                   activation="swigluoai", w1_bias=ex.w13_bias.data.cpu(),
+                                   w2_bias=ex.w2_bias.data.cpu(), mirror_rounding=True)
+    _close(out, ref)

@@ -219,3 +219,59 @@ def test_fused_gate_topk_falls_back_and_block_matches_two_step(moe, oracle, dev,
     full = oracle.fused_experts_ref(flat.cpu(), blk.experts.w13_weight.data.cpu(),
                                     blk.experts.w2_weight.data.cpu(), tw.cpu(), tids.cpu())
     assert (out.view(-1, H).float().cpu() - full).abs().max() < 1e-2 + 2e-2 * full.abs().max()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("T,H", [(1, 8), (7, 2048), (300, 2048), (64, 4096), (33, 1000), (5, 8192), (3, 12288)])
+def test_add_rms_norm_against_oracle(moe, oracle, dev, dtype, T, H):
+    """csrc/layernorm_kernels.cu:77-108 / :10-35: the residual sum is bit-exact (one fp32
+    add, one rounding); the normalised output is rounded twice (before and after the
+    weight), so against the float64-variance oracle it may differ by two rounding steps of
+    the dtype where the fp32 reduction lands on the other side of a tie."""
+    g = torch.Generator().manual_seed(T * 131 + H)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    res = (torch.randn(T, H, generator=g) * 3).to(dtype)
+    w = (1.0 + 0.2 * torch.randn(H, generator=g)).to(dtype)
+    step = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10, torch.float32: 2.0 ** -21}[dtype]
+    want, want_res = oracle.add_rms_norm(x, res, w, 1e-6)
+    out = torch.empty(T, H, dtype=dtype, device=dev)
+    res_d = res.to(dev)
+    moe.ops.add_rms_norm(out, res_d, x.to(dev), w.to(dev), 1e-6)
+    assert torch.equal(res_d.cpu(), want_res)
+    diff = (out.cpu().double() - want.double()).abs()
+    assert (diff <= 2 * step * want.double().abs() + 1e-30).all()
+    if dtype != torch.float32:
+        assert (diff > 0).double().mean() < 0.02
+    # without a residual; strided rows (a column slice of a wider tensor) and in place
+    want2, _ = oracle.add_rms_norm(x, None, w, 1e-5)
+    wide = torch.zeros(T, H + 16, dtype=dtype, device=dev)
+    xin = wide[:, 8:8 + H]
+    xin.copy_(x)
+    moe.ops.rms_norm(xin, xin, w.to(dev), 1e-5)
+    diff2 = (xin.cpu().double() - want2.double()).abs()
+    assert (diff2 <= 2 * step * want2.double().abs() + 1e-30).all()
+    assert torch.count_nonzero(wide[:, :8]) == 0 and torch.count_nonzero(wide[:, 8 + H:]) == 0
+
+
+@pytest.mark.gpu
+def test_rms_norm_module_mirrors_the_reference_interface(moe, oracle, dev):
+    """nanovllm/layers/layernorm.py:7-34: forward(x) -> out; forward(x, residual) ->
+    (out, residual) with the residual updated in place."""
+    g = torch.Generator().manual_seed(5)
+    norm = moe.RMSNorm(512, eps=1e-6).to(dev).to(torch.bfloat16)
+    norm.weight.data.copy_((1.0 + 0.1 * torch.randn(512, generator=g)).bfloat16())
+    x = torch.randn(40, 512, generator=g).bfloat16()
+    res = torch.randn(40, 512, generator=g).bfloat16()
+    res_d = res.to(dev)
+    out, res_back = norm(x.to(dev), res_d)
+    assert res_back is res_d
+    want, want_res = oracle.add_rms_norm(x, res, norm.weight.data.cpu(), 1e-6)
+    assert torch.equal(res_d.cpu(), want_res)
+    assert ((out.cpu().double() - want.double()).abs() <= 2.0 ** -7 * want.double().abs()).all()
+    out1 = norm(x.to(dev))
+    want1, _ = oracle.add_rms_norm(x, None, norm.weight.data.cpu(), 1e-6)
+    assert ((out1.cpu().double() - want1.double()).abs() <= 2.0 ** -7 * want1.double().abs()).all()
+    with pytest.raises(RuntimeError, match="hidden_size"):
+        moe.ops.rms_norm(torch.empty(2, 4, 8, device=dev), torch.empty(2, 4, 8, device=dev),
+                         torch.ones(8, device=dev), 1e-6)

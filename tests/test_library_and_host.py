@@ -67,8 +67,12 @@ def test_argument_validation_without_gpu(moe):
     for rows, cols in ((67584 + 128 * 127, 768), (67584, 2048)):
         want += -(-rows * cols * 2 // 256) * 256
     assert L.moe_fused_experts_workspace_bytes(8448, 2048, 768, 128, 8, 128, 2, 2) == want
-    for m, bm in ((256, 32), (768, 64), (8448, 256)):
+    # act dtype code 2 = bf16: streaming blocks, then the large tile from 48 rows per expert on
+    for m, bm in ((256, 32), (512, 64), (768, 256), (8448, 256)):
         assert L.moe_preferred_block_size(m, 128, 8, 2, 2) == bm
+    # fp32 (code 0) has no large-tile kernel: the M tile follows the load
+    for m, bm in ((256, 32), (768, 64), (2048, 128), (8448, 256)):
+        assert L.moe_preferred_block_size(m, 128, 8, 0, 0) == bm
 
 
 def test_ops_refuse_cpu_tensors(moe):

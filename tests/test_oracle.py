@@ -348,3 +348,41 @@ def test_gate_logits_are_the_float64_linear_rounded_once(oracle):
         tw, ids, _ = oracle.gate_topk_softmax(x, w, 4, renormalize=True)
         tw2, ids2, _ = oracle.topk_softmax(got, 4, renormalize=True)
         assert torch.equal(ids, ids2) and torch.equal(tw, tw2)
+
+
+def test_add_rms_norm_known_answers(oracle):
+    """Pins the norm oracle on rows whose answer is exact: a dropped residual, a
+    variance taken over the wrong values or a missing weight each break one."""
+    # s = (3, 4): mean square 12.5, r = 1/sqrt(12.5); the residual carries half of the row
+    x = torch.tensor([[3.0, 0.0]])
+    res = torch.tensor([[0.0, 4.0]])
+    w = torch.tensor([2.0, 0.5])
+    out, new_res = oracle.add_rms_norm(x, res, w, 0.0)
+    assert torch.equal(new_res, torch.tensor([[3.0, 4.0]]))
+    r = 1.0 / (12.5 ** 0.5)
+    assert torch.allclose(out, torch.tensor([[3.0 * r * 2.0, 4.0 * r * 0.5]]), rtol=1e-6, atol=0)
+    # constant rows: x / |x| * w, exactly, for any power-of-two magnitude
+    for c in (0.5, -2.0, 8.0):
+        out, _ = oracle.add_rms_norm(torch.full((3, 16), c), None, torch.arange(16.0), 0.0)
+        assert torch.equal(out, torch.arange(16.0).expand(3, 16) * (1.0 if c > 0 else -1.0))
+    # eps enters under the root: zero rows give zero, tiny rows are damped
+    out, _ = oracle.add_rms_norm(torch.zeros(2, 8), None, torch.ones(8), 1e-6)
+    assert torch.equal(out, torch.zeros(2, 8))
+    out, _ = oracle.add_rms_norm(torch.full((1, 4), 1e-3), None, torch.ones(4), 1e-6)
+    assert torch.allclose(out, torch.full((1, 4), 1e-3 / (2e-6 ** 0.5)), rtol=1e-6)
+    # 16-bit dtypes: the sum is rounded into the residual, the variance is not
+    xb = torch.tensor([[1.0, 2.0 ** -8]], dtype=torch.bfloat16)
+    rb = torch.tensor([[2.0 ** -8, 1.0]], dtype=torch.bfloat16)
+    out, new_res = oracle.add_rms_norm(xb, rb, torch.ones(2, dtype=torch.bfloat16), 0.0)
+    assert torch.equal(new_res, torch.ones(1, 2, dtype=torch.bfloat16))     # 1 + 2^-8 rounds (to even) to 1 in bf16
+    assert torch.equal(out, torch.full((1, 2), 1.0 - 2.0 ** -8).to(torch.bfloat16))  # r = 1/(1 + 2^-8), not 1
+    # against the float64 textbook formula on random rows, one rounding step at most
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(32, 256, generator=g).bfloat16()
+    res = torch.randn(32, 256, generator=g).bfloat16()
+    w = (1.0 + 0.1 * torch.randn(256, generator=g)).bfloat16()
+    out, new_res = oracle.add_rms_norm(x, res, w, 1e-6)
+    s64 = x.double() + res.double()
+    assert torch.equal(new_res, s64.to(torch.bfloat16))
+    want = new_res.double() / torch.sqrt((s64 * s64).mean(-1, keepdim=True) + 1e-6) * w.double()
+    assert ((out.double() - want).abs() <= 2.0 ** -7 * want.abs() + 1e-12).all()
