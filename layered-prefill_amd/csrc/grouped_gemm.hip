@@ -135,6 +135,7 @@ struct GemmParams {
   int64_t sorted_cap; // capacity of sorted_ids
   int align_bs;      // block size the alignment was made with (a multiple of the kernel's M tile)
   int m_major;       // workgroup order inside an XCD: all n-tiles of an m-block are neighbours
+  const int32_t* xcd_bounds;  // large-tile kernel: m-block range [b[x], b[x+1]) of XCD x, or null
 };
 
 constexpr int kThreads = 256;
@@ -639,6 +640,76 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
 #endif
 }
 
+// Main loop for tiles with at most 64 real slots (an expert that received only a
+// few rows): nothing but weight streaming, so the ring is laid out for that.
+// Four 32 KB weight units (ring slots 1, 3, 0, 2 in that order, so that W(0) and
+// W(1), requested by the caller before it knew the count, are where they
+// belong) and four 8 KB token units of 64 rows inside slot 4.  Three K tiles are
+// in flight while one is multiplied, twice what the general loop keeps in flight
+// for weights, and a token unit costs two requests per wavefront instead of eight.
+template <typename Mma, int FMC>
+__device__ __forceinline__ void big_light_mainloop(const BigCtx& c, const char* smem, int nk,
+                                                   f32x16 (&acc)[4][4]) {
+  static_assert(FMC <= 2, "at most 64 token rows");
+  constexpr int CH = Mma::kBigChunks, STEPS = 4 / CH;
+  constexpr int kTokUnit = 2 * 4096;  // 64 rows
+  auto w_slot = [](int k) {
+    const int q = k & 3;
+    return (q == 0 ? 1 : q == 1 ? 3 : q == 2 ? 0 : 2) * kBigUnitBytes;
+  };
+  auto a_slot = [](int k) { return 4 * kBigUnitBytes + (k & 3) * kTokUnit; };
+  auto issue_w = [&](int k) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) lds_dma16(c.w_base + k * kBigRowBytes, c.w_off[i], c.dma_lds + w_slot(k) + i * 4096);
+  };
+  auto issue_a = [&](int k) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) lds_dma16(c.a_base + k * kBigRowBytes, c.a_off[i], c.dma_lds + a_slot(k) + i * 4096);
+  };
+  // request order: W(0) W(1) (caller) A(0) A(1) W(2) A(2), then W(k) A(k) per K tile
+  issue_a(0);
+  if (1 < nk) issue_a(1);
+  if (2 < nk) { issue_w(2); issue_a(2); }
+  for (int kt = 0; kt < nk; ++kt) {
+    // unit kt has landed: only the (up to two) younger units may be outstanding; and
+    // this wavefront is done reading unit kt-1, whose slots the next requests reuse
+    const int left = nk - 1 - kt;
+    if (kt == 0) {
+      if (left >= 2) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");
+      else if (left == 1) asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    } else {
+      if (left >= 2) asm volatile("s_waitcnt vmcnt(20) lgkmcnt(0)" ::: "memory");
+      else if (left == 1) asm volatile("s_waitcnt vmcnt(10) lgkmcnt(0)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    }
+    bare_barrier();
+    if (kt + 3 < nk) { issue_w(kt + 3); issue_a(kt + 3); }
+    if constexpr (FMC > 0) {
+      const char* sw = smem + w_slot(kt);
+      const char* sa = smem + a_slot(kt);
+#pragma unroll
+      for (int kk = 0; kk < STEPS; ++kk) {
+        uint4 wf[4][CH], xf[FMC][CH];
+#pragma unroll
+        for (int ch = 0; ch < CH; ++ch) {
+#pragma unroll
+          for (int fm = 0; fm < FMC; ++fm)
+            xf[fm][ch] = *reinterpret_cast<const uint4*>(sa + fm * 32 * kBigRowBytes + c.rd_k[kk * CH + ch]);
+#pragma unroll
+          for (int fn = 0; fn < 4; ++fn)
+            wf[fn][ch] = *reinterpret_cast<const uint4*>(sw + c.w_row[fn] + c.rd_k[kk * CH + ch]);
+        }
+#pragma unroll
+        for (int fm = 0; fm < FMC; ++fm)
+#pragma unroll
+          for (int fn = 0; fn < 4; ++fn) acc[fn][fm] = Mma::mma_big(wf[fn], xf[fm], acc[fn][fm]);
+      }
+    }
+  }
+  wait_vmcnt<0>();
+}
+
 // Epilogue phase 1: round this wavefront's accumulators to the activation dtype
 // (after the optional bias and routed weight) and park them in its LDS window
 // as [token row][weight row].
@@ -807,7 +878,7 @@ __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, i
   }
 }
 
-template <typename Mma, int FMC, bool GATED>
+template <typename Mma, int FMC, bool GATED, bool LIGHT = false>
 __device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, char* smem, int nk,
                                          int e, int n0, int wn, int wm, int lane, int my_tok, float my_rw,
                                          float my_as, int* s_tok_all, float* s_rw_all, char* epi) {
@@ -819,7 +890,8 @@ __device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, c
     for (int fm = 0; fm < 4; ++fm)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[fn][fm][r] = 0.f;
-  big_mainloop<Mma, FMC>(c, smem, nk, acc);
+  if constexpr (LIGHT) big_light_mainloop<Mma, FMC>(c, smem, nk, acc);
+  else big_mainloop<Mma, FMC>(c, smem, nk, acc);
 #ifdef MOE_TRACE
   if (threadIdx.x == 0 && blockIdx.x < 4096) moe_dbg[blockIdx.x * 8 + 7] = MOE_TRACE_NOW();
 #endif
@@ -846,20 +918,28 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   extern __shared__ __attribute__((aligned(16))) char smem[];
   // only the m-blocks below the padded total are live: cut the per-XCD ranges from
   // those, so that no XCD is left holding the grid's empty tail
+  const int xslot = blockIdx.x / kXcds;
+  int nt, mb;
+  if (p.xcd_bounds) {
+    // ranges of equal estimated work (big_plan_kernel), m-block major inside a range
+    const int lo = p.xcd_bounds[blockIdx.x % kXcds], hi = p.xcd_bounds[blockIdx.x % kXcds + 1];
+    mb = lo + xslot / p.num_n_tiles;
+    nt = xslot % p.num_n_tiles;
+    if (mb >= hi) return;
+  } else {
   const int npp = *p.num_post_pad;
   const int live_mb = (npp + kBigBM - 1) / kBigBM;
   const int live = live_mb * p.num_n_tiles;
   const int per_xcd = (live + kXcds - 1) / kXcds;
-  const int xslot = blockIdx.x / kXcds;
   const int logical = (blockIdx.x % kXcds) * per_xcd + xslot;
   if (xslot >= per_xcd || logical >= live) return;
-  int nt, mb;
   if (p.m_major) {
     mb = logical / p.num_n_tiles;
     nt = logical - mb * p.num_n_tiles;
   } else {
     nt = logical / live_mb;
     mb = logical - nt * live_mb;
+  }
   }
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lhi = lane >> 5;
@@ -953,6 +1033,14 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   [[maybe_unused]] const unsigned long long t_pro = MOE_TRACE_NOW();
   const int rows = min(128, max(0, nvalid - wm * 128));  // real slots of this wavefront
   __syncthreads();  // s_tok sits inside the ring: everyone has read it before any DMA may land there
+  if (nvalid <= 64) {
+    // a workgroup-wide choice: every wavefront runs the streaming-shaped loop
+    switch ((rows + 31) >> 5) {
+      case 0: big_wave<Mma, 0, GATED, true>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, s_tok, s_rw_all, epi); break;
+      case 1: big_wave<Mma, 1, GATED, true>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, s_tok, s_rw_all, epi); break;
+      default: big_wave<Mma, 2, GATED, true>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, s_tok, s_rw_all, epi); break;
+    }
+  } else
   switch ((rows + 31) >> 5) {
     case 0: big_wave<Mma, 0, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, s_tok, s_rw_all, epi); break;
     case 1: big_wave<Mma, 1, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, s_tok, s_rw_all, epi); break;
@@ -983,6 +1071,81 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
 #endif
 }
 
+
+// Cuts the live m-blocks of a large-tile launch into one contiguous range per XCD
+// with equal estimated work instead of equal counts.  A block of an expert that
+// received at most 32 (64) rows is weight streaming only and costs about 0.53
+// (0.69) of a full one; with equal counts the XCDs finished up to 25 % apart.
+// Ranges stay contiguous so that the blocks of one expert keep sharing its
+// weights through one L2.  No range is longer than cap_mb blocks (the grid has
+// that many slots per XCD).  One workgroup; bounds[0..8] in m-blocks.
+constexpr int kPlanThreads = 1024;
+__global__ __launch_bounds__(kPlanThreads) void big_plan_kernel(const int32_t* __restrict__ sorted_ids,
+                                                                const int32_t* __restrict__ num_post_pad,
+                                                                int numel, int cap_mb, int32_t* __restrict__ bounds) {
+  __shared__ int s_wave[kPlanThreads / kWave + 1];
+  __shared__ int s_b[kXcds + 1];
+  const int live_mb = (*num_post_pad + kBigBM - 1) / kBigBM;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  auto weight = [&](int mb) {
+    if (mb >= live_mb) return 0;
+    const int32_t* s = sorted_ids + static_cast<int64_t>(mb) * kBigBM;
+    return s[32] >= numel ? 17 : (s[64] >= numel ? 22 : 32);
+  };
+  // inclusive scan of `v` over the workgroup, plus the workgroup total
+  auto scan = [&](int v, int& total) {
+    int inc = v;
+#pragma unroll
+    for (int d = 1; d < kWave; d *= 2) {
+      const int o = __shfl_up(inc, d, kWave);
+      if (lane >= d) inc += o;
+    }
+    __syncthreads();
+    if (lane == kWave - 1) s_wave[wave] = inc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int run = 0;
+      for (int w = 0; w < kPlanThreads / kWave; ++w) { const int t = s_wave[w]; s_wave[w] = run; run += t; }
+      s_wave[kPlanThreads / kWave] = run;
+    }
+    __syncthreads();
+    total = s_wave[kPlanThreads / kWave];
+    return inc + s_wave[wave];
+  };
+  int total = 0;
+  for (int base = 0; base < live_mb; base += kPlanThreads) {
+    int t;
+    scan(weight(base + threadIdx.x), t);
+    total += t;
+  }
+  if (threadIdx.x <= kXcds) s_b[threadIdx.x] = threadIdx.x == 0 ? 0 : live_mb;
+  __syncthreads();
+  int before = 0;
+  for (int base = 0; base < live_mb; base += kPlanThreads) {
+    const int mb = base + threadIdx.x;
+    const int w = weight(mb);
+    int t;
+    const int inc = before + scan(w, t), exc = inc - w;
+    if (w > 0) {
+      // the block whose cost takes the running sum across x / 8 of the total is the last of XCD x - 1
+#pragma unroll
+      for (int x = 1; x < kXcds; ++x) {
+        const int64_t target = (static_cast<int64_t>(total) * x + kXcds - 1) / kXcds;
+        if (exc < target && inc >= target) s_b[x] = mb + 1;
+      }
+    }
+    before += t;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    // a total of 0 (no live block) leaves every bound at live_mb = 0; otherwise bounds ascend
+    for (int x = 1; x <= kXcds; ++x) s_b[x] = max(s_b[x], s_b[x - 1]);
+    for (int x = 1; x <= kXcds; ++x) s_b[x] = min(s_b[x], s_b[x - 1] + cap_mb);
+    s_b[kXcds] = live_mb;
+    for (int x = kXcds - 1; x >= 1; --x) s_b[x] = max(s_b[x], s_b[x + 1] - cap_mb);
+    for (int x = 0; x <= kXcds; ++x) bounds[x] = s_b[x];
+  }
+}
 
 // Epilogue of the streaming kernel for full, aligned 16-bit tiles: same storage
 // points as store_fragment, with the hardware conversions and the fast SiLU of
@@ -1225,6 +1388,14 @@ int launch_stream(GemmParams& p, int64_t sorted_cap, hipStream_t s) {
   return moe_check_launch(GATED ? "fused_experts (gate-up pass)" : "fused_experts (down pass)");
 }
 
+// Longest m-block range big_plan_kernel may give an XCD: twice the average (a range of
+// weight-streaming blocks only, at about half the cost each), never more than all blocks.
+static int big_plan_cap(int64_t sorted_cap) {
+  const int64_t mbs = (sorted_cap + kBigBM - 1) / kBigBM;
+  const int64_t cap = 2 * ((mbs + kXcds - 1) / kXcds);
+  return static_cast<int>(cap < mbs ? cap : mbs);
+}
+
 template <typename Mma, bool GATED>
 int launch_big(GemmParams& p, int64_t sorted_cap, hipStream_t s) {
   constexpr int lds = kBigLdsTotal;
@@ -1240,7 +1411,9 @@ int launch_big(GemmParams& p, int64_t sorted_cap, hipStream_t s) {
   p.num_m_blocks = static_cast<int>((sorted_cap + kBigBM - 1) / kBigBM);
   p.num_n_tiles = (p.N + (GATED ? 128 : 256) - 1) / (GATED ? 128 : 256);
   const int64_t tiles = static_cast<int64_t>(p.num_m_blocks) * p.num_n_tiles;
-  const int64_t grid = (tiles + kXcds - 1) / kXcds * kXcds;
+  int64_t grid = (tiles + kXcds - 1) / kXcds * kXcds;
+  if (p.xcd_bounds)  // work-balanced ranges: as many slots per XCD as the longest range may have blocks
+    grid = static_cast<int64_t>(big_plan_cap(sorted_cap)) * p.num_n_tiles * kXcds;
   if (grid > INT32_MAX) return moe_fail(MOE_ERR_ARG, "fused_experts: grid of %lld workgroups", static_cast<long long>(grid));
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(kThreads), lds, s, p);
   return moe_check_launch(GATED ? "fused_experts (gate-up pass)" : "fused_experts (down pass)");
@@ -1275,16 +1448,20 @@ template <typename Mma, bool GATED>
 int launch_bm(GemmParams& p, int block_size, int64_t sorted_cap, hipStream_t s) {
   p.align_bs = block_size;
   p.m_major = 0;
+  const int32_t* bounds = p.xcd_bounds;  // meant for the large-tile kernel only
+  p.xcd_bounds = nullptr;
   if constexpr (Mma::kEs == 1) {
     // a large-tile K step is 128 bytes per row: 128 e4m3 elements
     if (block_size % 256 == 0 && p.Kd % kBigRowBytes == 0) {
       p.m_major = 1;
+      p.xcd_bounds = bounds;
       return launch_big<MmaE4M3Big<typename Mma::El>, GATED>(p, sorted_cap, s);
     }
   }
   if constexpr (Mma::kEs == 2) {
     if (block_size % 256 == 0 && p.Kd % kBigBK == 0) {
       p.m_major = 1;  // a token block is reused by all its n-tiles through one L2
+      p.xcd_bounds = bounds;
       return launch_big<Mma, GATED>(p, sorted_cap, s);
     }
     // byte offsets of token rows are 32-bit in the streaming kernel
@@ -1308,6 +1485,15 @@ int launch_bm(GemmParams& p, int block_size, int64_t sorted_cap, hipStream_t s) 
     return launch<Mma, 32, 256, 1, GATED>(p, s);
   }
   return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: block_size %d is not a multiple of 32", block_size);
+}
+
+bool plan_enabled() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("MOE_BIG_PLAN");
+    v = (e && e[0] == '0') ? 0 : 1;
+  }
+  return v == 1;
 }
 
 int elem_size(int dtype) { return dtype == MOE_F32 ? 4 : (dtype == MOE_E4M3 ? 1 : 2); }
@@ -1345,7 +1531,7 @@ MOE_EXPORT int64_t moe_fused_experts_workspace_bytes(int T, int H, int I, int E,
   if (weight_dtype == MOE_E4M3)  // e4m3 copies of x and of the intermediate, one fp32 scale per row
     bytes += moe_align_up(static_cast<int64_t>(T) * H, 256) + moe_align_up(static_cast<int64_t>(T) * 4, 256) +
              moe_align_up(rows * I, 256) + moe_align_up(rows * 4, 256);
-  return bytes;
+  return bytes + 256;  // per-XCD m-block ranges of the large-tile kernel
 }
 
 MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
@@ -1411,6 +1597,16 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.limit = a->swiglu_limit;
   p.activation = a->activation;
   p.interleaved = a->activation == MOE_ACT_SWIGLUOAI;
+  const int32_t* plan_bounds = nullptr;
+  if (a->block_size % kBigBM == 0 && a->act_dtype != MOE_F32 && plan_enabled()) {
+    // both passes walk the same m-blocks: one plan for the two launches
+    int32_t* bounds = reinterpret_cast<int32_t*>(static_cast<char*>(a->workspace) + need_ws - 256);
+    hipLaunchKernelGGL(big_plan_kernel, dim3(1), dim3(kPlanThreads), 0, s, a->sorted_token_ids,
+                       a->num_tokens_post_pad, static_cast<int>(numel), big_plan_cap(a->sorted_cap), bounds);
+    if (int rc0 = moe_check_launch("fused_experts (XCD ranges)")) return rc0;
+    plan_bounds = bounds;
+  }
+  p.xcd_bounds = plan_bounds;
   // pass 1: x . W13^T with the gated activation, rows addressed by slot
   p.a = a->x; p.lda = a->H; p.w = a->w13; p.w_stride_e = a->w13_stride_e; p.w_stride_n = a->w13_stride_n;
   p.bias = a->w13_bias; p.bias_stride_e = 2LL * a->I;
@@ -1437,6 +1633,7 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.bias = a->w2_bias; p.bias_stride_e = a->H;
   p.c = c3; p.ldc = a->H; p.Kd = a->I; p.N = a->H; p.a_by_slot = 1;
   p.mul_weight = a->apply_router_weight_on_input ? 0 : 1;
+  p.xcd_bounds = plan_bounds;
   if (fp8 && (passes & 2)) {
     // the activated intermediate is quantised per slot row the same way
     rc = moe_quant_rows_e4m3(inter, a->act_dtype, rows, a->I, reinterpret_cast<uint8_t*>(iq), is, a->stream);
