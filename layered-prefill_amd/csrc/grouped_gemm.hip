@@ -411,7 +411,7 @@ constexpr int kBigDmaPerUnit = 8;                  // global_load_lds instructio
 constexpr int kEpiRowBytes = 128 * 2 + 16;   // one token row of a wavefront's tile, padded
 constexpr int kEpiWaveBytes = 128 * kEpiRowBytes;
 constexpr int kBigLdsBytes = 4 * kEpiWaveBytes;    // epilogue staging, reuses the ring
-constexpr int kBigSideBytes = 4 * kBigBM * 4;      // per slot: token id, routed weight, fp8 row scale; per weight row: fp8 scale
+constexpr int kBigSideBytes = 5 * kBigBM * 4;      // per slot: token id, routed weight, fp8 row scale; per weight row: fp8 scale, bias
 constexpr int kBigLdsTotal = kBigUnits * kBigUnitBytes;  // the whole 160 KB of the CU
 static_assert(kBigLdsBytes + kBigSideBytes + 16 <= kBigLdsTotal, "epilogue staging must fit in the ring");
 
@@ -715,26 +715,11 @@ __device__ __forceinline__ void big_light_mainloop(const BigCtx& c, const char* 
 // as [token row][weight row].
 template <typename El, int FMC, bool GATED, bool SCALED, bool BIAS>
 __device__ __forceinline__ void big_park(const GemmParams& p, int e, int n0, int wn, int lhi, int l32,
-                                         const float* s_rw, const float* s_as, const float* s_ws, char* epi,
-                                         const f32x16 (&acc)[4][4]) {
-  using S = typename El::S;
-  const S* bias = static_cast<const S*>(p.bias);
-  // weight row (output channel) behind accumulator element (fn, 4 * g + i) of this lane
-  auto wrow_of = [&](int fn, int g, int i) -> int64_t {
-    const int local = fn * 32 + 8 * g + 4 * lhi + i;  // column inside the wavefront tile
-    if constexpr (GATED) {
-      int col = n0 + wn * 64 + (local & 63);
-      col = col < p.N ? col : p.N - 1;
-      const int half = local >> 6;
-      return p.interleaved ? 2 * col + half : half * p.N + col;
-    } else {
-      const int col = n0 + wn * 128 + local;
-      return col < p.N ? col : p.N - 1;
-    }
-  };
+                                         const float* s_rw, const float* s_as, const float* s_ws,
+                                         const float* s_bias, char* epi, const f32x16 (&acc)[4][4]) {
   // e4m3: the accumulator is in units of (row scale of the A operand) x (weight row scale)
-  // e4m3: the accumulator is in units of (row scale of the A operand) x (weight row scale);
-  // the weight rows' scales were put into LDS in the order of the weight unit's rows
+  // e4m3: the accumulator is in units of (row scale of the A operand) x (weight row scale).
+  // Scales and biases of the weight rows were put into LDS in the order of the weight unit's rows.
   [[maybe_unused]] int ws_row[4];
 #pragma unroll
   for (int fn = 0; fn < 4; ++fn) {
@@ -758,8 +743,8 @@ __device__ __forceinline__ void big_park(const GemmParams& p, int e, int n0, int
           v[0] *= as * w4.x; v[1] *= as * w4.y; v[2] *= as * w4.z; v[3] *= as * w4.w;
         }
         if constexpr (BIAS) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) v[i] += El::ld(bias[e * p.bias_stride_e + wrow_of(fn, g, i)]);
+          const float4 b4 = *reinterpret_cast<const float4*>(s_bias + ws_row[fn] + 8 * g + 4 * lhi);
+          v[0] += b4.x; v[1] += b4.y; v[2] += b4.z; v[3] += b4.w;
         }
         // rw is exactly 1 when the routed weight is not applied in this pass
 #pragma unroll
@@ -882,7 +867,7 @@ __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, i
 template <typename Mma, int FMC, bool GATED, bool LIGHT = false>
 __device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, char* smem, int nk,
                                          int e, int n0, int wn, int wm, int lane, int my_tok, float my_rw,
-                                         float my_as, float my_ws, int* s_tok_all, float* s_rw_all, char* epi) {
+                                         float my_as, float my_ws, float my_bias, int* s_tok_all, float* s_rw_all, char* epi) {
   using El = typename Mma::El;
   f32x16 acc[4][4];
 #pragma unroll
@@ -901,16 +886,17 @@ __device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, c
   s_rw_all[threadIdx.x] = my_rw;  // requested before the main loop, needed only now
   s_rw_all[kBigBM + threadIdx.x] = my_as;
   s_rw_all[2 * kBigBM + threadIdx.x] = my_ws;
+  s_rw_all[3 * kBigBM + threadIdx.x] = my_bias;
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   bare_barrier();
   if constexpr (FMC > 0) {
     // one straight-line body per case: a test per element costs more than the element
     if (p.bias)
       big_park<El, FMC, GATED, Mma::kEs == 1, true>(p, e, n0, wn, lane >> 5, lane & 31, s_rw_all + wm * 128,
-                                                    s_rw_all + kBigBM + wm * 128, s_rw_all + 2 * kBigBM, epi, acc);
+                                                    s_rw_all + kBigBM + wm * 128, s_rw_all + 2 * kBigBM, s_rw_all + 3 * kBigBM, epi, acc);
     else
       big_park<El, FMC, GATED, Mma::kEs == 1, false>(p, e, n0, wn, lane >> 5, lane & 31, s_rw_all + wm * 128,
-                                                     s_rw_all + kBigBM + wm * 128, s_rw_all + 2 * kBigBM, epi, acc);
+                                                     s_rw_all + kBigBM + wm * 128, s_rw_all + 2 * kBigBM, s_rw_all + 3 * kBigBM, epi, acc);
   }
 }
 
@@ -1002,8 +988,9 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   float my_rw = 1.f, my_as = 1.f, my_ws = 1.f;
   if (p.mul_weight) my_rw = my_tok < p.numel ? p.topk_w[my_tok] : 0.f;
   if (p.a_scale && my_tok < p.numel) my_as = p.a_scale[p.a_by_slot ? my_slot : my_tok / p.top_k];
-  if (p.w_scale) {
-    // scale of the weight row that sits at row `tid` of a weight unit
+  float my_bias = 0.f;
+  if (p.w_scale || p.bias) {
+    // scale and bias of the weight row that sits at row `tid` of a weight unit
     int64_t wr;
     if constexpr (GATED) {
       int n = n0 + (tid & 127);
@@ -1012,7 +999,8 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
     } else {
       wr = n0 + tid < p.N ? n0 + tid : p.N - 1;
     }
-    my_ws = p.w_scale[e * p.w_scale_stride_e + wr];
+    if (p.w_scale) my_ws = p.w_scale[e * p.w_scale_stride_e + wr];
+    if (p.bias) my_bias = El::ld(static_cast<const typename El::S*>(p.bias)[e * p.bias_stride_e + wr]);
   }
   const int a_groups = (nvalid + 31) >> 5;  // 32-row token groups that hold real slots
 #pragma unroll
@@ -1050,17 +1038,17 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   if (nvalid <= 64) {
     // a workgroup-wide choice: every wavefront runs the streaming-shaped loop
     switch ((rows + 31) >> 5) {
-      case 0: big_wave<Mma, 0, GATED, true>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, s_tok, s_rw_all, epi); break;
-      case 1: big_wave<Mma, 1, GATED, true>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, s_tok, s_rw_all, epi); break;
-      default: big_wave<Mma, 2, GATED, true>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, s_tok, s_rw_all, epi); break;
+      case 0: big_wave<Mma, 0, GATED, true>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, my_bias, s_tok, s_rw_all, epi); break;
+      case 1: big_wave<Mma, 1, GATED, true>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, my_bias, s_tok, s_rw_all, epi); break;
+      default: big_wave<Mma, 2, GATED, true>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, my_bias, s_tok, s_rw_all, epi); break;
     }
   } else
   switch ((rows + 31) >> 5) {
-    case 0: big_wave<Mma, 0, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, s_tok, s_rw_all, epi); break;
-    case 1: big_wave<Mma, 1, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, s_tok, s_rw_all, epi); break;
-    case 2: big_wave<Mma, 2, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, s_tok, s_rw_all, epi); break;
-    case 3: big_wave<Mma, 3, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, s_tok, s_rw_all, epi); break;
-    default: big_wave<Mma, 4, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, s_tok, s_rw_all, epi); break;
+    case 0: big_wave<Mma, 0, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, my_bias, s_tok, s_rw_all, epi); break;
+    case 1: big_wave<Mma, 1, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, my_bias, s_tok, s_rw_all, epi); break;
+    case 2: big_wave<Mma, 2, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, my_bias, s_tok, s_rw_all, epi); break;
+    case 3: big_wave<Mma, 3, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, my_bias, s_tok, s_rw_all, epi); break;
+    default: big_wave<Mma, 4, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, my_bias, s_tok, s_rw_all, epi); break;
   }
   [[maybe_unused]] const unsigned long long t_main = MOE_TRACE_NOW();
   if constexpr (GATED) {
