@@ -13,6 +13,11 @@ int moe_fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)
 // Checks hipGetLastError() after a launch; 0 or MOE_ERR_LAUNCH.
 int moe_check_launch(const char* what);
 
+// moe_quant_rows_e4m3 restricted to the live slots of an expert-sorted matrix (library-internal).
+int moe_quant_slot_rows_e4m3(const void* w, int src_dtype, int64_t rows, int cols, uint8_t* q,
+                             float* scales, const int32_t* row_ids, int64_t id_count, int numel,
+                             void* stream);
+
 static inline int64_t moe_align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
 constexpr int kWave = 64;

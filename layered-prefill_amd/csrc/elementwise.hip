@@ -99,10 +99,11 @@ __device__ __forceinline__ uint8_t f32_to_e4m3(float v) {
 template <typename El>
 __global__ __launch_bounds__(kThreads) void quant_rows_e4m3_kernel(
     const typename El::S* __restrict__ w, int64_t rows, int cols, uint8_t* __restrict__ q,
-    float* __restrict__ scales) {
+    float* __restrict__ scales, const int32_t* __restrict__ row_ids, int64_t id_count, int numel) {
   const int lane = threadIdx.x % kWave;
   const int64_t row = blockIdx.x * static_cast<int64_t>(kThreads / kWave) + threadIdx.x / kWave;
   if (row >= rows) return;
+  if (row_ids && (row >= id_count || row_ids[row] >= numel)) return;  // a padding slot: nobody reads it
   const typename El::S* src = w + row * cols;
   float amax = 0.f;
   for (int c = lane; c < cols; c += kWave) amax = fmaxf(amax, fabsf(El::ld(src[c])));
@@ -119,10 +120,11 @@ __global__ __launch_bounds__(kThreads) void quant_rows_e4m3_kernel(
 template <typename El, int NV>
 __global__ __launch_bounds__(kThreads) void quant_rows_e4m3_vec_kernel(
     const typename El::S* __restrict__ w, int64_t rows, int cols, uint8_t* __restrict__ q,
-    float* __restrict__ scales) {
+    float* __restrict__ scales, const int32_t* __restrict__ row_ids, int64_t id_count, int numel) {
   const int lane = threadIdx.x % kWave;
   const int64_t row = blockIdx.x * static_cast<int64_t>(kThreads / kWave) + threadIdx.x / kWave;
   if (row >= rows) return;
+  if (row_ids && (row >= id_count || row_ids[row] >= numel)) return;  // a padding slot: nobody reads it
   const uint4* src = reinterpret_cast<const uint4*>(w + row * cols);
   const int nvec = cols / 8;
   uint4 v[NV];
@@ -160,16 +162,16 @@ __global__ __launch_bounds__(kThreads) void quant_rows_e4m3_vec_kernel(
 }
 
 template <typename El>
-bool launch_quant_vec(const void* w, int64_t rows, int cols, uint8_t* q, float* scales, dim3 grid,
-                      hipStream_t s) {
+bool launch_quant_vec(const void* w, int64_t rows, int cols, uint8_t* q, float* scales,
+                      const int32_t* row_ids, int64_t id_count, int numel, dim3 grid, hipStream_t s) {
   using S = typename El::S;
   if (cols % 8 != 0 || cols > 4096 || (reinterpret_cast<uintptr_t>(w) & 15u) || (reinterpret_cast<uintptr_t>(q) & 7u))
     return false;
   const int nv = (cols / 8 + kWave - 1) / kWave;
   const S* src = static_cast<const S*>(w);
-  if (nv <= 2) hipLaunchKernelGGL((quant_rows_e4m3_vec_kernel<El, 2>), grid, dim3(kThreads), 0, s, src, rows, cols, q, scales);
-  else if (nv <= 4) hipLaunchKernelGGL((quant_rows_e4m3_vec_kernel<El, 4>), grid, dim3(kThreads), 0, s, src, rows, cols, q, scales);
-  else hipLaunchKernelGGL((quant_rows_e4m3_vec_kernel<El, 8>), grid, dim3(kThreads), 0, s, src, rows, cols, q, scales);
+  if (nv <= 2) hipLaunchKernelGGL((quant_rows_e4m3_vec_kernel<El, 2>), grid, dim3(kThreads), 0, s, src, rows, cols, q, scales, row_ids, id_count, numel);
+  else if (nv <= 4) hipLaunchKernelGGL((quant_rows_e4m3_vec_kernel<El, 4>), grid, dim3(kThreads), 0, s, src, rows, cols, q, scales, row_ids, id_count, numel);
+  else hipLaunchKernelGGL((quant_rows_e4m3_vec_kernel<El, 8>), grid, dim3(kThreads), 0, s, src, rows, cols, q, scales, row_ids, id_count, numel);
   return true;
 }
 
@@ -270,6 +272,14 @@ MOE_EXPORT int moe_sum(void* out, const void* in, int64_t T, int K, int H, int d
 
 MOE_EXPORT int moe_quant_rows_e4m3(const void* w, int src_dtype, int64_t rows, int cols,
                                    uint8_t* q, float* scales, void* stream) {
+  return moe_quant_slot_rows_e4m3(w, src_dtype, rows, cols, q, scales, nullptr, 0, 0, stream);
+}
+
+// Row r is skipped (q and scales left untouched) when row_ids is given and r >= id_count or
+// row_ids[r] >= numel: the padding slots of an expert-sorted intermediate.
+int moe_quant_slot_rows_e4m3(const void* w, int src_dtype, int64_t rows, int cols, uint8_t* q,
+                             float* scales, const int32_t* row_ids, int64_t id_count, int numel,
+                             void* stream) {
   if (rows < 0 || cols < 1) return moe_fail(MOE_ERR_ARG, "quant_rows_e4m3: bad sizes rows=%lld cols=%d", static_cast<long long>(rows), cols);
   if (rows == 0) return MOE_OK;
   if (!w || !q || !scales) return moe_fail(MOE_ERR_ARG, "quant_rows_e4m3: null pointer");
@@ -279,15 +289,15 @@ MOE_EXPORT int moe_quant_rows_e4m3(const void* w, int src_dtype, int64_t rows, i
   const dim3 grid(static_cast<unsigned>(blocks)), block(kThreads);
   switch (src_dtype) {
     case MOE_F32:
-      hipLaunchKernelGGL(quant_rows_e4m3_kernel<ElemF32>, grid, block, 0, s, static_cast<const float*>(w), rows, cols, q, scales);
+      hipLaunchKernelGGL(quant_rows_e4m3_kernel<ElemF32>, grid, block, 0, s, static_cast<const float*>(w), rows, cols, q, scales, row_ids, id_count, numel);
       break;
     case MOE_F16:
-      if (!launch_quant_vec<ElemF16>(w, rows, cols, q, scales, grid, s))
-        hipLaunchKernelGGL(quant_rows_e4m3_kernel<ElemF16>, grid, block, 0, s, static_cast<const uint16_t*>(w), rows, cols, q, scales);
+      if (!launch_quant_vec<ElemF16>(w, rows, cols, q, scales, row_ids, id_count, numel, grid, s))
+        hipLaunchKernelGGL(quant_rows_e4m3_kernel<ElemF16>, grid, block, 0, s, static_cast<const uint16_t*>(w), rows, cols, q, scales, row_ids, id_count, numel);
       break;
     case MOE_BF16:
-      if (!launch_quant_vec<ElemBF16>(w, rows, cols, q, scales, grid, s))
-        hipLaunchKernelGGL(quant_rows_e4m3_kernel<ElemBF16>, grid, block, 0, s, static_cast<const uint16_t*>(w), rows, cols, q, scales);
+      if (!launch_quant_vec<ElemBF16>(w, rows, cols, q, scales, row_ids, id_count, numel, grid, s))
+        hipLaunchKernelGGL(quant_rows_e4m3_kernel<ElemBF16>, grid, block, 0, s, static_cast<const uint16_t*>(w), rows, cols, q, scales, row_ids, id_count, numel);
       break;
     default:
       return moe_fail(MOE_ERR_ARG, "quant_rows_e4m3: unsupported source dtype code %d", src_dtype);

@@ -717,7 +717,6 @@ template <typename El, int FMC, bool GATED, bool SCALED, bool BIAS>
 __device__ __forceinline__ void big_park(const GemmParams& p, int e, int n0, int wn, int lhi, int l32,
                                          const float* s_rw, const float* s_as, const float* s_ws,
                                          const float* s_bias, char* epi, const f32x16 (&acc)[4][4]) {
-  // e4m3: the accumulator is in units of (row scale of the A operand) x (weight row scale)
   // e4m3: the accumulator is in units of (row scale of the A operand) x (weight row scale).
   // Scales and biases of the weight rows were put into LDS in the order of the weight unit's rows.
   [[maybe_unused]] int ws_row[4];
@@ -1638,7 +1637,8 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.xcd_bounds = plan_bounds;
   if (fp8 && (passes & 2)) {
     // the activated intermediate is quantised per slot row the same way
-    rc = moe_quant_rows_e4m3(inter, a->act_dtype, rows, a->I, reinterpret_cast<uint8_t*>(iq), is, a->stream);
+    rc = moe_quant_slot_rows_e4m3(inter, a->act_dtype, rows, a->I, reinterpret_cast<uint8_t*>(iq), is,
+                                  a->sorted_token_ids, a->sorted_cap, static_cast<int>(numel), a->stream);
     if (rc) return rc;
     p.a = iq; p.a_scale = is; p.w_scale = a->w2_scale; p.w_scale_stride_e = a->H;
     rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaE4M3<ElemBF16>, false>(p, a->block_size, a->sorted_cap, s)
