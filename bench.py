@@ -33,8 +33,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE runs (profiles/hbm_traffic_gate_up_kernels.txt): fetch + write bytes.
-MEASURED_TRAFFIC_BYTES = {"layered_8192p_256d": 1742591386 + 106979328,
-                          "decode_256": 571216077 + 3341517}
+MEASURED_TRAFFIC_BYTES = {"layered_8192p_256d": 1773152256 + 114690048,
+                          "decode_256": 571137843 + 3340083}
 
 
 def _events(n):
