@@ -1488,15 +1488,6 @@ int launch_bm(GemmParams& p, int block_size, int64_t sorted_cap, hipStream_t s) 
   return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: block_size %d is not a multiple of 32", block_size);
 }
 
-bool plan_enabled() {
-  static int v = -1;
-  if (v < 0) {
-    const char* e = getenv("MOE_BIG_PLAN");
-    v = (e && e[0] == '0') ? 0 : 1;
-  }
-  return v == 1;
-}
-
 int elem_size(int dtype) { return dtype == MOE_F32 ? 4 : (dtype == MOE_E4M3 ? 1 : 2); }
 
 }  // namespace
@@ -1599,7 +1590,7 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.activation = a->activation;
   p.interleaved = a->activation == MOE_ACT_SWIGLUOAI;
   const int32_t* plan_bounds = nullptr;
-  if (a->block_size % kBigBM == 0 && a->act_dtype != MOE_F32 && plan_enabled()) {
+  if (a->block_size % kBigBM == 0 && a->act_dtype != MOE_F32) {
     // both passes walk the same m-blocks: one plan for the two launches
     int32_t* bounds = reinterpret_cast<int32_t*>(static_cast<char*>(a->workspace) + need_ws - 256);
     hipLaunchKernelGGL(big_plan_kernel, dim3(1), dim3(kPlanThreads), 0, s, a->sorted_token_ids,
