@@ -333,7 +333,8 @@ def main() -> int:
     ap.add_argument("--workload", default="layered_8192p_256d",
                     choices=["layered_8192p_256d", "decode_256"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-runs", type=int, default=2)
+    ap.add_argument("--cpu-runs", type=int, default=16,
+                    help="timed passes of the CPU baseline (about 0.65 s each on 16 cores)")
     ap.add_argument("--chunk-mode", default="both", choices=["both", "chunked", "single", "off"],
                     help="config 4 (chunk amplification) leg: both sides, one side only (for "
                          "rocprofv3 counter runs), or off")
