@@ -210,10 +210,19 @@ __global__ __launch_bounds__(kScanThreads) void align_scan_kernel(
   const int e = threadIdx.x % E, r = threadIdx.x / E;
   const bool active = r < R;
   const int sbeg = r * L, send = min(nseg, sbeg + L);
+  // counts are fetched eight at a time: issued one by one, each load would wait for the one before
+  constexpr int CH = 8;
   int sum = 0;
-  if (active)
-    for (int sg = sbeg; sg < send; ++sg) sum += seg_cnt[static_cast<size_t>(sg) * E + e];
-  if (active) s_part[r * E + e] = sum;
+  if (active) {
+    for (int sg0 = sbeg; sg0 < send; sg0 += CH) {
+      int c[CH];
+#pragma unroll
+      for (int i = 0; i < CH; ++i) c[i] = sg0 + i < send ? seg_cnt[static_cast<size_t>(sg0 + i) * E + e] : 0;
+#pragma unroll
+      for (int i = 0; i < CH; ++i) sum += c[i];
+    }
+    s_part[r * E + e] = sum;
+  }
   __syncthreads();
   if (active) {
     int running = 0, total = 0;
@@ -223,11 +232,15 @@ __global__ __launch_bounds__(kScanThreads) void align_scan_kernel(
       total += v;
     }
     if (r == 0) s_tot[e] = total;
-    for (int sg = sbeg; sg < send; ++sg) {
-      const size_t at = static_cast<size_t>(sg) * E + e;
-      const int c = seg_cnt[at];
-      seg_cnt[at] = running;
-      running += c;
+    for (int sg0 = sbeg; sg0 < send; sg0 += CH) {
+      int c[CH];
+#pragma unroll
+      for (int i = 0; i < CH; ++i) c[i] = sg0 + i < send ? seg_cnt[static_cast<size_t>(sg0 + i) * E + e] : 0;
+#pragma unroll
+      for (int i = 0; i < CH; ++i) {
+        if (sg0 + i < send) seg_cnt[static_cast<size_t>(sg0 + i) * E + e] = running;
+        running += c[i];
+      }
     }
   }
   __syncthreads();
