@@ -1451,23 +1451,26 @@ int launch_bm(GemmParams& p, int block_size, int64_t sorted_cap, hipStream_t s) 
   p.m_major = 0;
   const int32_t* bounds = p.xcd_bounds;  // meant for the large-tile kernel only
   p.xcd_bounds = nullptr;
+  // The DMA kernels address rows with 32-bit byte offsets from a 64-bit base: both
+  // operands must span less than 4 GiB (per expert, for the weights).
+  const int64_t a_rows = p.a_by_slot ? sorted_cap : p.numel / p.top_k;
+  const int64_t w_rows = GATED ? 2LL * p.N : p.N;
+  const bool offsets_fit = a_rows * p.lda * Mma::kEs < (1LL << 32) && w_rows * p.w_stride_n * Mma::kEs < (1LL << 32);
   if constexpr (Mma::kEs == 1) {
     // a large-tile K step is 128 bytes per row: 128 e4m3 elements
-    if (block_size % 256 == 0 && p.Kd % kBigRowBytes == 0) {
+    if (block_size % 256 == 0 && p.Kd % kBigRowBytes == 0 && offsets_fit) {
       p.m_major = 1;
       p.xcd_bounds = bounds;
       return launch_big<MmaE4M3Big<typename Mma::El>, GATED>(p, sorted_cap, s);
     }
   }
   if constexpr (Mma::kEs == 2) {
-    if (block_size % 256 == 0 && p.Kd % kBigBK == 0) {
+    if (block_size % 256 == 0 && p.Kd % kBigBK == 0 && offsets_fit) {
       p.m_major = 1;  // a token block is reused by all its n-tiles through one L2
       p.xcd_bounds = bounds;
       return launch_big<Mma, GATED>(p, sorted_cap, s);
     }
-    // byte offsets of token rows are 32-bit in the streaming kernel
-    const int64_t a_rows = p.a_by_slot ? sorted_cap : p.numel / p.top_k;
-    if (block_size == kStBM && p.Kd % kStBK == 0 && a_rows * p.lda * 2 < (1LL << 32))
+    if (block_size == kStBM && p.Kd % kStBK == 0 && offsets_fit)
       return launch_stream<Mma, GATED>(p, sorted_cap, s);
   }
   if (block_size % 128 == 0) {
