@@ -798,7 +798,7 @@ __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, i
   constexpr int COLS = GATED ? 64 : 128;      // output columns of the wavefront tile
   constexpr int LPR = COLS / 8;               // lanes per row
   constexpr int RPS = kWave / LPR;            // rows per step
-  constexpr int UNR = 4;                      // steps in flight: LDS reads, math and stores overlap
+  constexpr int UNR = GATED ? 4 : 8;          // steps in flight: LDS reads, math and stores overlap
   const int c8 = (lane % LPR) * 8;
   const int ncol = n0 + wn * COLS + c8;
   const bool vec_ok = ncol + 7 < p.N && (p.ldc & 7) == 0;
