@@ -394,3 +394,33 @@ def test_gpt_oss_mlp_block(moe, oracle, dev):
                                    activation="swigluoai", w1_bias=ex.w13_bias.data.cpu(),
                                    w2_bias=ex.w2_bias.data.cpu(), mirror_rounding=True)
     _close(out, ref)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("pattern", ["one_expert", "one_row_each", "two_heavy_rest_single"])
+def test_large_tile_ranges_on_lopsided_routing(moe, oracle, dev, pattern, monkeypatch):
+    """Alignment blocks of 256 with routings that make the per-XCD work ranges degenerate: every
+    block of one expert (ranges cut inside it), one row per expert (weight-streaming blocks
+    only), two heavy experts among many single-row ones (ranges of very unequal length)."""
+    E, H, I, K = 64, 256, 128, 1
+    g = torch.Generator().manual_seed(31)
+    if pattern == "one_expert":
+        T = 3000
+        ids = torch.full((T, 1), 5, dtype=torch.int32)
+    elif pattern == "one_row_each":
+        T = E
+        ids = torch.randperm(E, generator=g).to(torch.int32).view(T, 1)
+    else:
+        T = 2 * 1500 + (E - 2)
+        ids = torch.cat([torch.full((1500,), 7), torch.full((1500,), 40),
+                         torch.tensor([e for e in range(E) if e not in (7, 40)])]).to(torch.int32)
+        ids = ids[torch.randperm(T, generator=g)].view(T, 1)
+    x = torch.randn(T, H, generator=g).bfloat16()
+    w13 = (torch.randn(E, 2 * I, H, generator=g) * 0.05).bfloat16()
+    w2 = (torch.randn(E, H, I, generator=g) * 0.05).bfloat16()
+    tw = torch.rand(T, K, generator=g) + 0.5
+    monkeypatch.setattr(moe.fused_moe, "try_get_optimal_moe_config", lambda *a, **k: {"BLOCK_SIZE_M": 256})
+    d = lambda t: t.to(dev)
+    out = moe.fused_experts(d(x), d(w13), d(w2), None, None, d(tw), d(ids))
+    ref = oracle.fused_experts_ref(x, w13, w2, tw, ids, mirror_rounding=True)
+    _close(out, ref, rtol=1.6e-2, atol=2e-3 + 4e-3 * ref.abs().max().item())
