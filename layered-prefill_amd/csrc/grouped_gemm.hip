@@ -710,54 +710,6 @@ __device__ __forceinline__ void big_light_mainloop(const BigCtx& c, const char* 
   wait_vmcnt<0>();
 }
 
-// Epilogue phase 1: round this wavefront's accumulators to the activation dtype
-// (after the optional bias and routed weight) and park them in its LDS window
-// as [token row][weight row].
-template <typename El, int FMC, bool GATED, bool SCALED, bool BIAS>
-__device__ __forceinline__ void big_park(const GemmParams& p, int e, int n0, int wn, int lhi, int l32,
-                                         const float* s_rw, const float* s_as, const float* s_ws,
-                                         const float* s_bias, char* epi, const f32x16 (&acc)[4][4]) {
-  // e4m3: the accumulator is in units of (row scale of the A operand) x (weight row scale).
-  // Scales and biases of the weight rows were put into LDS in the order of the weight unit's rows.
-  [[maybe_unused]] int ws_row[4];
-#pragma unroll
-  for (int fn = 0; fn < 4; ++fn) {
-    if constexpr (GATED) ws_row[fn] = (fn < 2) ? wn * 64 + fn * 32 : 128 + wn * 64 + (fn - 2) * 32;
-    else ws_row[fn] = wn * 128 + fn * 32;
-  }
-#pragma unroll
-  for (int fm = 0; fm < FMC; ++fm) {
-    const float rw = s_rw[fm * 32 + l32];  // 1 when the routed weight is not applied here
-    [[maybe_unused]] const float as = SCALED ? s_as[fm * 32 + l32] : 1.f;
-    char* row = epi + (fm * 32 + l32) * kEpiRowBytes;
-#pragma unroll
-    for (int fn = 0; fn < 4; ++fn) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        float v[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = acc[fn][fm][4 * g + i];
-        if constexpr (SCALED) {
-          const float4 w4 = *reinterpret_cast<const float4*>(s_ws + ws_row[fn] + 8 * g + 4 * lhi);
-          v[0] *= as * w4.x; v[1] *= as * w4.y; v[2] *= as * w4.z; v[3] *= as * w4.w;
-        }
-        if constexpr (BIAS) {
-          const float4 b4 = *reinterpret_cast<const float4*>(s_bias + ws_row[fn] + 8 * g + 4 * lhi);
-          v[0] += b4.x; v[1] += b4.y; v[2] += b4.z; v[3] += b4.w;
-        }
-        // rw is exactly 1 when the routed weight is not applied in this pass
-#pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] *= rw;
-        *reinterpret_cast<uint2*>(row + (fn * 32 + 8 * g + 4 * lhi) * 2) =
-            uint2{pack2<El>(v[0], v[1]), pack2<El>(v[2], v[3])};
-      }
-    }
-  }
-}
-
-// Epilogue phase 2: write the parked tile to global memory, 8 columns (16 bytes)
-// per lane and step.  Gated: columns [0,64) of a row are gate values, [64,128)
-// the matching up values.
 template <typename El>
 __device__ __forceinline__ float unpack_lo(uint32_t w);
 template <typename El>
@@ -791,6 +743,70 @@ __device__ __forceinline__ uint32_t gated_pair(const GemmParams& p, uint32_t gw,
   }
 }
 
+// Epilogue phase 1: park this wavefront's results in its LDS window as
+// [token row][weight row], rounded to the activation dtype after the optional
+// scales, bias and routed weight.  FAST_SILU (gated pass with SiLU): gate row n
+// and up row n of the weight unit are the same accumulator element of fragments
+// fn and fn + 2, so silu(gate) * up is formed here on the fp32 values (hardware
+// exp2/rcp, one rounding at the end) and only the 64 output columns are parked.
+// The other activations park gate and up rounded, as the stand-alone activation
+// kernels see them, and the flush combines them.
+template <typename El, int FMC, bool GATED, bool SCALED, bool BIAS, bool FAST_SILU>
+__device__ __forceinline__ void big_park(const GemmParams& p, int e, int n0, int wn, int lhi, int l32,
+                                         const float* s_rw, const float* s_as, const float* s_ws,
+                                         const float* s_bias, char* epi, const f32x16 (&acc)[4][4]) {
+  // e4m3: the accumulator is in units of (row scale of the A operand) x (weight row scale).
+  // Scales and biases of the weight rows were put into LDS in the order of the weight unit's rows.
+  [[maybe_unused]] int ws_row[4];
+#pragma unroll
+  for (int fn = 0; fn < 4; ++fn) {
+    if constexpr (GATED) ws_row[fn] = (fn < 2) ? wn * 64 + fn * 32 : 128 + wn * 64 + (fn - 2) * 32;
+    else ws_row[fn] = wn * 128 + fn * 32;
+  }
+  // four consecutive accumulator elements of fragment fn, scaled, biased, weighted
+  auto load4 = [&](int fn, int fm, int g, float as, float rw, float (&v)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = acc[fn][fm][4 * g + i];
+    if constexpr (SCALED) {
+      const float4 w4 = *reinterpret_cast<const float4*>(s_ws + ws_row[fn] + 8 * g + 4 * lhi);
+      v[0] *= as * w4.x; v[1] *= as * w4.y; v[2] *= as * w4.z; v[3] *= as * w4.w;
+    }
+    if constexpr (BIAS) {
+      const float4 b4 = *reinterpret_cast<const float4*>(s_bias + ws_row[fn] + 8 * g + 4 * lhi);
+      v[0] += b4.x; v[1] += b4.y; v[2] += b4.z; v[3] += b4.w;
+    }
+    // rw is exactly 1 when the routed weight is not applied in this pass
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] *= rw;
+  };
+#pragma unroll
+  for (int fm = 0; fm < FMC; ++fm) {
+    const float rw = s_rw[fm * 32 + l32];
+    [[maybe_unused]] const float as = SCALED ? s_as[fm * 32 + l32] : 1.f;
+    char* row = epi + (fm * 32 + l32) * kEpiRowBytes;
+#pragma unroll
+    for (int fn = 0; fn < (FAST_SILU ? 2 : 4); ++fn) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float v[4];
+        load4(fn, fm, g, as, rw, v);
+        if constexpr (FAST_SILU) {
+          float u[4];
+          load4(fn + 2, fm, g, as, rw, u);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] = silu_fast(v[i]) * u[i];
+        }
+        *reinterpret_cast<uint2*>(row + (fn * 32 + 8 * g + 4 * lhi) * 2) =
+            uint2{pack2<El>(v[0], v[1]), pack2<El>(v[2], v[3])};
+      }
+    }
+  }
+}
+
+// Epilogue phase 2: write the parked tile to global memory, 8 columns (16 bytes)
+// per lane and step.  After a gated pass with SiLU the 64 output columns of a
+// row are parked ready; with the other activations columns [0,64) of a row are
+// gate values and [64,128) the matching up values, combined here.
 template <typename El, bool GATED, int ACT>
 __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, int lane, int slot0,
                                           int rows, const int* s_tok, const char* epi) {
@@ -798,7 +814,8 @@ __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, i
   constexpr int COLS = GATED ? 64 : 128;      // output columns of the wavefront tile
   constexpr int LPR = COLS / 8;               // lanes per row
   constexpr int RPS = kWave / LPR;            // rows per step
-  constexpr int UNR = GATED ? 4 : 8;          // steps in flight: LDS reads, math and stores overlap
+  constexpr bool PAIRS = GATED && ACT != MOE_ACT_SILU;  // gate and up parked side by side, activation applied here
+  constexpr int UNR = PAIRS ? 4 : 8;          // steps in flight: LDS reads, math and stores overlap
   const int c8 = (lane % LPR) * 8;
   const int ncol = n0 + wn * COLS + c8;
   const bool vec_ok = ncol + 7 < p.N && (p.ldc & 7) == 0;
@@ -817,12 +834,12 @@ __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, i
         const int r = r0 + u * RPS + lrow;  // < 128: rows <= 128 and 128 is a multiple of RPS * UNR
         crow[u] = p.a_by_slot ? s_tok[r] : slot0 + r;
         gq[u] = *reinterpret_cast<const uint4*>(src + (r0 + u * RPS) * kEpiRowBytes);
-        if constexpr (GATED) uq[u] = *reinterpret_cast<const uint4*>(src + (r0 + u * RPS) * kEpiRowBytes + 128);
+        if constexpr (PAIRS) uq[u] = *reinterpret_cast<const uint4*>(src + (r0 + u * RPS) * kEpiRowBytes + 128);
       }
 #pragma unroll
       for (int u = 0; u < UNR; ++u) {
         uint4 out = gq[u];
-        if constexpr (GATED)
+        if constexpr (PAIRS)
           out = uint4{gated_pair<El, ACT>(p, gq[u].x, uq[u].x), gated_pair<El, ACT>(p, gq[u].y, uq[u].y),
                       gated_pair<El, ACT>(p, gq[u].z, uq[u].z), gated_pair<El, ACT>(p, gq[u].w, uq[u].w)};
         if (r0 + u * RPS + lrow < rows) *reinterpret_cast<uint4*>(cbase + crow[u] * ldc_bytes) = out;
@@ -839,13 +856,13 @@ __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, i
       tok[u] = r < rows ? s_tok[r] : p.numel;
       const char* row = epi + (r < 128 ? r : 127) * kEpiRowBytes;
       gq[u] = *reinterpret_cast<const uint4*>(row + c8 * 2);
-      if constexpr (GATED) uq[u] = *reinterpret_cast<const uint4*>(row + (64 + c8) * 2);
+      if constexpr (PAIRS) uq[u] = *reinterpret_cast<const uint4*>(row + (64 + c8) * 2);
     }
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
       if (tok[u] >= p.numel) continue;
       uint4 out = gq[u];
-      if constexpr (GATED)
+      if constexpr (PAIRS)
         out = uint4{gated_pair<El, ACT>(p, gq[u].x, uq[u].x), gated_pair<El, ACT>(p, gq[u].y, uq[u].y),
                     gated_pair<El, ACT>(p, gq[u].z, uq[u].z), gated_pair<El, ACT>(p, gq[u].w, uq[u].w)};
       const int slot = slot0 + r0 + u * RPS + lane / LPR;
@@ -890,12 +907,23 @@ __device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, c
   bare_barrier();
   if constexpr (FMC > 0) {
     // one straight-line body per case: a test per element costs more than the element
-    if (p.bias)
-      big_park<El, FMC, GATED, Mma::kEs == 1, true>(p, e, n0, wn, lane >> 5, lane & 31, s_rw_all + wm * 128,
-                                                    s_rw_all + kBigBM + wm * 128, s_rw_all + 2 * kBigBM, s_rw_all + 3 * kBigBM, epi, acc);
-    else
-      big_park<El, FMC, GATED, Mma::kEs == 1, false>(p, e, n0, wn, lane >> 5, lane & 31, s_rw_all + wm * 128,
-                                                     s_rw_all + kBigBM + wm * 128, s_rw_all + 2 * kBigBM, s_rw_all + 3 * kBigBM, epi, acc);
+    auto park = [&](auto bias_tag, auto silu_tag) {
+      big_park<El, FMC, GATED, Mma::kEs == 1, decltype(bias_tag)::value != 0, decltype(silu_tag)::value != 0>(
+          p, e, n0, wn, lane >> 5, lane & 31, s_rw_all + wm * 128, s_rw_all + kBigBM + wm * 128,
+          s_rw_all + 2 * kBigBM, s_rw_all + 3 * kBigBM, epi, acc);
+    };
+    bool fast_silu = false;
+    if constexpr (GATED) fast_silu = p.activation == MOE_ACT_SILU;
+    if constexpr (GATED) {
+      if (fast_silu) {
+        if (p.bias) park(IntTag<1>{}, IntTag<1>{});
+        else park(IntTag<0>{}, IntTag<1>{});
+      }
+    }
+    if (!fast_silu) {
+      if (p.bias) park(IntTag<1>{}, IntTag<0>{});
+      else park(IntTag<0>{}, IntTag<0>{});
+    }
   }
 }
 
@@ -1051,7 +1079,6 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
   }
   [[maybe_unused]] const unsigned long long t_main = MOE_TRACE_NOW();
   if constexpr (GATED) {
-    // one tight loop per activation instead of a three-way branch per element
     if (p.activation == MOE_ACT_SILU)
       big_flush<El, true, MOE_ACT_SILU>(p, n0, wn, lane, slot0, rows, s_tok + wm * 128, epi);
     else if (p.activation == MOE_ACT_SWIGLUOAI)

@@ -251,7 +251,7 @@ def fused_experts_ref(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.T
                       activation: str = "silu", apply_router_weight_on_input: bool = False,
                       w1_bias: Optional[torch.Tensor] = None,
                       w2_bias: Optional[torch.Tensor] = None,
-                      mirror_rounding: bool = False,
+                      mirror_rounding=False,
                       out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """out[t] = sum_k w[t,k] * W2[e] @ act(W13[e] @ x_t), e = ids[t,k].
 
@@ -261,9 +261,13 @@ def fused_experts_ref(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.T
     silu, after the gate*up product, after the routed-weight multiply, after
     the top-k sum; nanovllm/layers/for_moe/fused_moe.py:216,522-531,
     csrc/activation_kernels.cu:11,23), fp32 accumulation in between.
+    ``mirror_rounding="fused"``: as ``True``, except that the SiLU-gated
+    intermediate is rounded once, where a kernel that applies the activation to
+    its fp32 accumulators stores it (no rounding after GEMM1 or after silu).
     """
     x = _cpu(hidden_states)
     dt = x.dtype if mirror_rounding else None
+    fused_act = mirror_rounding == "fused" and activation == "silu"
     T, H = x.shape
     E, N, _ = w1.shape
     K = topk_ids.shape[1]
@@ -281,12 +285,12 @@ def fused_experts_ref(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.T
             c1 = c1 + _cpu(w1_bias[e]).float()                # :207-208
         if apply_router_weight_on_input:
             c1 = c1 * tw[tok, slot, None]                     # :210-214 via :589
-        c1 = _round(c1, dt)                                   # :216
+        c1 = _round(c1, None if fused_act else dt)            # :216
         if activation == "silu":
-            if dt is None:
+            if dt is None or fused_act:
                 d = N // 2
                 g, u = c1[:, :d], c1[:, d:]
-                c2 = g / (1 + torch.exp(-g)) * u
+                c2 = _round(g / (1 + torch.exp(-g)) * u, dt)
             else:
                 c2 = silu_and_mul(c1.to(dt)).float()
         elif activation == "swigluoai":
@@ -310,7 +314,7 @@ def fused_experts_ref(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.T
 def fused_experts_fp8_ref(hidden_states: torch.Tensor, w1_q: torch.Tensor, w1_scale: torch.Tensor,
                           w2_q: torch.Tensor, w2_scale: torch.Tensor,
                           topk_weights: torch.Tensor, topk_ids: torch.Tensor,
-                          mirror_rounding: bool = False) -> torch.Tensor:
+                          mirror_rounding=False) -> torch.Tensor:
     """fp32 reference of the fp8 variant (not implemented by the reference:
     nanovllm/layers/for_moe/fused_moe.py:248-249,571,607 assert the scales are
     None): e4m3 per-output-channel weights, dynamic per-token e4m3 activations
@@ -319,9 +323,11 @@ def fused_experts_fp8_ref(hidden_states: torch.Tensor, w1_q: torch.Tensor, w1_sc
     ``mirror_rounding=True`` additionally rounds to the activation dtype where
     the bf16 path stores an intermediate (GEMM1 result, silu, silu*up, weighted
     GEMM2 result, top-k sum), i.e. the second quantisation sees the stored
-    16-bit intermediate rather than its fp32 value."""
+    16-bit intermediate rather than its fp32 value.  ``mirror_rounding="fused"``
+    rounds that intermediate once (no rounding after GEMM1 or after silu)."""
     x16 = _cpu(hidden_states)
     dt = x16.dtype if mirror_rounding else None
+    fused_act = mirror_rounding == "fused"
     x = x16.float()
     T, H = x.shape
     E, N, _ = w1_q.shape
@@ -339,10 +345,10 @@ def fused_experts_fp8_ref(hidden_states: torch.Tensor, w1_q: torch.Tensor, w1_sc
         W1 = dequant_e4m3(w1_q[e]) * _cpu(w1_scale[e]).float()[:, None]
         W2 = dequant_e4m3(w2_q[e]) * _cpu(w2_scale[e]).float()[:, None]
         c1 = xd[tok] @ W1.t()
-        if dt is None:
+        if dt is None or fused_act:
             d = N // 2
             g, u = c1[:, :d], c1[:, d:]
-            c2 = g / (1 + torch.exp(-g)) * u
+            c2 = _round(g / (1 + torch.exp(-g)) * u, dt)
         else:
             c2 = silu_and_mul(c1.to(dt)).float()
         cq, cs = quant_act_per_token(c2)

@@ -330,6 +330,14 @@ def test_mirrored_rounding_stays_close_to_fp32(oracle):
     a = oracle.fused_experts_ref(x, w13, w2, w, ids)
     b = oracle.fused_experts_ref(x, w13, w2, w, ids, mirror_rounding=True)
     assert torch.allclose(a, b, rtol=2e-2, atol=1e-2)
+    # one rounding of the gated intermediate instead of three: between the two
+    c = oracle.fused_experts_ref(x, w13, w2, w, ids, mirror_rounding="fused")
+    assert torch.allclose(a, c, rtol=2e-2, atol=1e-2) and not torch.equal(b, c)
+    assert (a - c).abs().mean() <= (a - b).abs().mean()
+    # with fp32 activations no mode rounds anything
+    xf, wf13, wf2 = x.float(), w13.float(), w2.float()
+    assert torch.equal(oracle.fused_experts_ref(xf, wf13, wf2, w, ids, mirror_rounding="fused"),
+                       oracle.fused_experts_ref(xf, wf13, wf2, w, ids))
 
 
 def test_gate_logits_are_the_float64_linear_rounded_once(oracle):
