@@ -143,7 +143,8 @@ typedef struct MoeFusedExpertsArgs {
   /* bit mask of the passes to enqueue: 1 gate-up GEMM + activation, 2 down GEMM
      times routed weight, 4 top-k combine; 0 means all three.  Lets a profiler
      or benchmark time one pass alone (the later passes then read whatever the
-     workspace holds). */
+     workspace holds).  Bit 8 keeps the two GEMM passes in separate launches
+     where the library would otherwise enqueue them as one. */
   int32_t passes;
   void* stream;
 } MoeFusedExpertsArgs;

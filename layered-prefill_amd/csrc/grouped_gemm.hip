@@ -927,35 +927,10 @@ __device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, c
   }
 }
 
+// One output tile of the large-tile kernel: m-block mb, n-tile nt.
 template <typename Mma, bool GATED>
-__global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams p) {
+__device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, char* smem) {
   using El = typename Mma::El;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  // only the m-blocks below the padded total are live: cut the per-XCD ranges from
-  // those, so that no XCD is left holding the grid's empty tail
-  const int xslot = blockIdx.x / kXcds;
-  int nt, mb;
-  if (p.xcd_bounds) {
-    // ranges of equal estimated work (big_plan_kernel), m-block major inside a range
-    const int lo = p.xcd_bounds[blockIdx.x % kXcds], hi = p.xcd_bounds[blockIdx.x % kXcds + 1];
-    mb = lo + xslot / p.num_n_tiles;
-    nt = xslot % p.num_n_tiles;
-    if (mb >= hi) return;
-  } else {
-  const int npp = *p.num_post_pad;
-  const int live_mb = (npp + kBigBM - 1) / kBigBM;
-  const int live = live_mb * p.num_n_tiles;
-  const int per_xcd = (live + kXcds - 1) / kXcds;
-  const int logical = (blockIdx.x % kXcds) * per_xcd + xslot;
-  if (xslot >= per_xcd || logical >= live) return;
-  if (p.m_major) {
-    mb = logical / p.num_n_tiles;
-    nt = logical - mb * p.num_n_tiles;
-  } else {
-    nt = logical / live_mb;
-    mb = logical - nt * live_mb;
-  }
-  }
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lhi = lane >> 5;
   const int wm = wave & 1, wn = wave >> 1;
@@ -1099,6 +1074,79 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
 #endif
 }
 
+template <typename Mma, bool GATED>
+__global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  // only the m-blocks below the padded total are live: cut the per-XCD ranges from
+  // those, so that no XCD is left holding the grid's empty tail
+  const int xslot = blockIdx.x / kXcds;
+  int nt, mb;
+  if (p.xcd_bounds) {
+    // ranges of equal estimated work (big_plan_kernel), m-block major inside a range
+    const int lo = p.xcd_bounds[blockIdx.x % kXcds], hi = p.xcd_bounds[blockIdx.x % kXcds + 1];
+    mb = lo + xslot / p.num_n_tiles;
+    nt = xslot % p.num_n_tiles;
+    if (mb >= hi) return;
+  } else {
+  const int npp = *p.num_post_pad;
+  const int live_mb = (npp + kBigBM - 1) / kBigBM;
+  const int live = live_mb * p.num_n_tiles;
+  const int per_xcd = (live + kXcds - 1) / kXcds;
+  const int logical = (blockIdx.x % kXcds) * per_xcd + xslot;
+  if (xslot >= per_xcd || logical >= live) return;
+  if (p.m_major) {
+    mb = logical / p.num_n_tiles;
+    nt = logical - mb * p.num_n_tiles;
+  } else {
+    nt = logical / live_mb;
+    mb = logical - nt * live_mb;
+  }
+  }
+  big_tile<Mma, GATED>(p, mb, nt, smem);
+}
+
+// Both passes in one launch, for the 16-bit dtypes.  Workgroup ids go to the XCDs
+// round robin and an XCD starts its workgroups in id order: each XCD first gets
+// the gate-up tiles of its m-block range, then the down tiles of the same range,
+// so its CUs move on to down tiles while the last gate-up tiles are still running
+// instead of idling through the tail of one launch and the ramp of the next.
+// A down tile reads intermediate rows that gate-up tiles of the same XCD wrote:
+// they meet in that XCD's L2.  done[mb] counts the finished gate-up tiles of
+// m-block mb (zeroed by big_plan_kernel); a down tile starts once all of them are
+// in, which at its place in the order is normally long the case.  The wait is
+// bounded (spin_limit polls of about a microsecond), so the grid drains even if
+// the order were not what is assumed.
+template <typename Mma>
+__global__ __launch_bounds__(kThreads, 1) void big_fused_kernel(const GemmParams p1, const GemmParams p2,
+                                                                int32_t* __restrict__ done, int cap_mb,
+                                                                int spin_limit) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int x = blockIdx.x % kXcds, xslot = blockIdx.x / kXcds;
+  const int lo = p1.xcd_bounds[x], hi = p1.xcd_bounds[x + 1];
+  const int n1 = cap_mb * p1.num_n_tiles;
+  if (xslot < n1) {
+    const int mb = lo + xslot / p1.num_n_tiles, nt = xslot % p1.num_n_tiles;
+    if (mb >= hi) return;
+    big_tile<Mma, true>(p1, mb, nt, smem);
+    // every store of this tile has been taken by the L2 before the count goes up
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) __hip_atomic_fetch_add(done + mb, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  } else {
+    const int j = xslot - n1;
+    const int mb = lo + j / p2.num_n_tiles, nt = j % p2.num_n_tiles;
+    if (mb >= hi) return;
+    if (threadIdx.x == 0) {
+      int spins = 0;
+      while (__hip_atomic_load(done + mb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < p1.num_n_tiles &&
+             spins++ < spin_limit)
+        __builtin_amdgcn_s_sleep(32);
+    }
+    __syncthreads();
+    big_tile<Mma, false>(p2, mb, nt, smem);
+  }
+}
+
 
 // Cuts the live m-blocks of a large-tile launch into one contiguous range per XCD
 // with equal estimated work instead of equal counts.  A block of an expert that
@@ -1110,8 +1158,11 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
 constexpr int kPlanThreads = 1024;
 __global__ __launch_bounds__(kPlanThreads) void big_plan_kernel(const int32_t* __restrict__ sorted_ids,
                                                                 const int32_t* __restrict__ num_post_pad,
-                                                                int numel, int cap_mb, int32_t* __restrict__ bounds) {
+                                                                int numel, int cap_mb, int32_t* __restrict__ bounds,
+                                                                int32_t* __restrict__ done, int num_done) {
   __shared__ int s_wave[kPlanThreads / kWave + 1];
+  // per-m-block counters of the one-launch form start at zero
+  for (int i = threadIdx.x; i < num_done; i += kPlanThreads) done[i] = 0;
   __shared__ int s_b[kXcds + 1];
   const int live_mb = (*num_post_pad + kBigBM - 1) / kBigBM;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -1472,17 +1523,57 @@ int launch(const GemmParams& p, hipStream_t s) {
 // else runs on the register-staged kernels with the largest M tile that
 // divides the block size, so that a block is a whole number of tiles of one
 // expert.
+// The DMA kernels address rows with 32-bit byte offsets from a 64-bit base: both
+// operands must span less than 4 GiB (per expert, for the weights).
+static bool dma_offsets_fit(const GemmParams& p, bool gated, int64_t sorted_cap, int es) {
+  const int64_t a_rows = p.a_by_slot ? sorted_cap : p.numel / p.top_k;
+  const int64_t w_rows = gated ? 2LL * p.N : p.N;
+  return a_rows * p.lda * es < (1LL << 32) && w_rows * p.w_stride_n * es < (1LL << 32);
+}
+
+// Whether a 16-bit pass runs on the large-tile kernel.
+static bool big_16bit_ok(const GemmParams& p, bool gated, int block_size, int64_t sorted_cap) {
+  return block_size % kBigBM == 0 && p.Kd % kBigBK == 0 && dma_offsets_fit(p, gated, sorted_cap, 2);
+}
+
+// Gate-up and down pass of the large-tile kernel in one launch (16-bit dtypes).
+// p1.xcd_bounds must be set; `done` holds one zeroed counter per m-block.
+template <typename Mma>
+int launch_big_fused(GemmParams& p1, GemmParams& p2, int block_size, int64_t sorted_cap, int32_t* done,
+                     hipStream_t s) {
+  constexpr int lds = kBigLdsTotal;
+  auto kern = big_fused_kernel<Mma>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess)
+      return moe_fail(MOE_ERR_LAUNCH, "fused_experts: cannot reserve %d B of LDS: %s", lds, hipGetErrorString(e));
+    attr_set = true;
+  }
+  for (GemmParams* q : {&p1, &p2}) {
+    q->align_bs = block_size;
+    q->m_major = 1;
+    q->num_m_blocks = static_cast<int>((sorted_cap + kBigBM - 1) / kBigBM);
+  }
+  p1.num_n_tiles = (p1.N + 127) / 128;
+  p2.num_n_tiles = (p2.N + 255) / 256;
+  const int cap_mb = big_plan_cap(sorted_cap);
+  const int64_t grid = static_cast<int64_t>(cap_mb) * (p1.num_n_tiles + p2.num_n_tiles) * kXcds;
+  if (grid > INT32_MAX) return moe_fail(MOE_ERR_ARG, "fused_experts: grid of %lld workgroups", static_cast<long long>(grid));
+  // a poll is about a microsecond: two seconds, far beyond any launch of this kernel
+  constexpr int kSpinLimit = 2000000;
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(kThreads), lds, s, p1, p2, done, cap_mb, kSpinLimit);
+  return moe_check_launch("fused_experts (gate-up and down pass, one launch)");
+}
+
 template <typename Mma, bool GATED>
 int launch_bm(GemmParams& p, int block_size, int64_t sorted_cap, hipStream_t s) {
   p.align_bs = block_size;
   p.m_major = 0;
   const int32_t* bounds = p.xcd_bounds;  // meant for the large-tile kernel only
   p.xcd_bounds = nullptr;
-  // The DMA kernels address rows with 32-bit byte offsets from a 64-bit base: both
-  // operands must span less than 4 GiB (per expert, for the weights).
-  const int64_t a_rows = p.a_by_slot ? sorted_cap : p.numel / p.top_k;
-  const int64_t w_rows = GATED ? 2LL * p.N : p.N;
-  const bool offsets_fit = a_rows * p.lda * Mma::kEs < (1LL << 32) && w_rows * p.w_stride_n * Mma::kEs < (1LL << 32);
+  const bool offsets_fit = dma_offsets_fit(p, GATED, sorted_cap, Mma::kEs);
   if constexpr (Mma::kEs == 1) {
     // a large-tile K step is 128 bytes per row: 128 e4m3 elements
     if (block_size % 256 == 0 && p.Kd % kBigRowBytes == 0 && offsets_fit) {
@@ -1492,7 +1583,7 @@ int launch_bm(GemmParams& p, int block_size, int64_t sorted_cap, hipStream_t s) 
     }
   }
   if constexpr (Mma::kEs == 2) {
-    if (block_size % 256 == 0 && p.Kd % kBigBK == 0 && offsets_fit) {
+    if (big_16bit_ok(p, GATED, block_size, sorted_cap)) {
       p.m_major = 1;  // a token block is reused by all its n-tiles through one L2
       p.xcd_bounds = bounds;
       return launch_big<Mma, GATED>(p, sorted_cap, s);
@@ -1553,7 +1644,9 @@ MOE_EXPORT int64_t moe_fused_experts_workspace_bytes(int T, int H, int I, int E,
   if (weight_dtype == MOE_E4M3)  // e4m3 copies of x and of the intermediate, one fp32 scale per row
     bytes += moe_align_up(static_cast<int64_t>(T) * H, 256) + moe_align_up(static_cast<int64_t>(T) * 4, 256) +
              moe_align_up(rows * I, 256) + moe_align_up(rows * 4, 256);
-  return bytes + 256;  // per-XCD m-block ranges of the large-tile kernel
+  // one counter per 256-slot block (one-launch form of the large-tile passes), then
+  // the per-XCD m-block ranges of the large-tile kernel
+  return bytes + moe_align_up((sorted_cap + kBigBM - 1) / kBigBM * 4, 256) + 256;
 }
 
 MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
@@ -1620,11 +1713,15 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.activation = a->activation;
   p.interleaved = a->activation == MOE_ACT_SWIGLUOAI;
   const int32_t* plan_bounds = nullptr;
+  int32_t* plan_done = nullptr;
   if (a->block_size % kBigBM == 0 && a->act_dtype != MOE_F32) {
     // both passes walk the same m-blocks: one plan for the two launches
     int32_t* bounds = reinterpret_cast<int32_t*>(static_cast<char*>(a->workspace) + need_ws - 256);
+    const int num_done = static_cast<int>((a->sorted_cap + kBigBM - 1) / kBigBM);
+    plan_done = bounds - moe_align_up(static_cast<int64_t>(num_done) * 4, 256) / 4;
     hipLaunchKernelGGL(big_plan_kernel, dim3(1), dim3(kPlanThreads), 0, s, a->sorted_token_ids,
-                       a->num_tokens_post_pad, static_cast<int>(numel), big_plan_cap(a->sorted_cap), bounds);
+                       a->num_tokens_post_pad, static_cast<int>(numel), big_plan_cap(a->sorted_cap), bounds,
+                       plan_done, num_done);
     if (int rc0 = moe_check_launch("fused_experts (XCD ranges)")) return rc0;
     plan_bounds = bounds;
   }
@@ -1636,6 +1733,21 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.mul_weight = a->apply_router_weight_on_input ? 1 : 0;
   const int passes = a->passes ? a->passes : 7;
   int rc = MOE_OK;
+  if (plan_bounds && !fp8 && (passes & 3) == 3 && !(passes & 8)) {
+    // 16-bit dtypes on the large-tile kernel: both passes in one launch
+    GemmParams p2 = p;
+    p2.a = inter; p2.lda = a->I; p2.w = a->w2; p2.w_stride_e = a->w2_stride_e; p2.w_stride_n = a->w2_stride_n;
+    p2.bias = a->w2_bias; p2.bias_stride_e = a->H;
+    p2.c = c3; p2.ldc = a->H; p2.Kd = a->I; p2.N = a->H; p2.a_by_slot = 1;
+    p2.mul_weight = a->apply_router_weight_on_input ? 0 : 1;
+    if (big_16bit_ok(p, true, a->block_size, a->sorted_cap) && big_16bit_ok(p2, false, a->block_size, a->sorted_cap)) {
+      rc = a->act_dtype == MOE_BF16 ? launch_big_fused<MmaBF16>(p, p2, a->block_size, a->sorted_cap, plan_done, s)
+                                    : launch_big_fused<MmaF16>(p, p2, a->block_size, a->sorted_cap, plan_done, s);
+      if (rc) return rc;
+      if (!(passes & 4)) return MOE_OK;
+      return moe_sum(a->out, c3, a->T, a->K, a->H, a->act_dtype, a->stream);
+    }
+  }
   if (fp8 && (passes & 1)) {
     // dynamic per-token e4m3 activations: s[t] = amax|x[t]| / 448
     rc = moe_quant_rows_e4m3(a->x, a->act_dtype, a->T, a->H, reinterpret_cast<uint8_t*>(xq), xs, a->stream);

@@ -141,7 +141,8 @@ def launch_fused_experts(x: torch.Tensor, out: torch.Tensor, w1: torch.Tensor, w
     tokens (the part of nanovllm/layers/for_moe/fused_moe.py:579-631 after
     moe_align_block_size).  ``workspace`` (uint8) is allocated when not given;
     ``passes`` selects single passes for profiling (1 gate-up, 2 down, 4
-    combine, 0 = all)."""
+    combine, 0 = all; adding 8 keeps the two GEMM passes in separate launches
+    where the library would enqueue them as one)."""
     T, H = x.shape
     E, N, _ = w1.shape
     top_k = topk_weights.shape[1]

@@ -434,3 +434,31 @@ def test_large_tile_ranges_on_lopsided_routing(moe, oracle, dev, pattern, monkey
     out = moe.fused_experts(d(x), d(w13), d(w2), None, None, d(tw), d(ids))
     _close_mirrored(out, lambda m: oracle.fused_experts_ref(x, w13, w2, tw, ids, mirror_rounding=m),
                     rtol=1.6e-2, atol=2e-3 + 4e-3 * out.float().abs().max().item())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("E,H,I,T,K,act", [(16, 512, 256, 2500, 4, "silu"), (8, 256, 192, 3000, 2, "swigluoai"),
+                                          (64, 256, 128, 6000, 8, "silu")])
+def test_one_launch_form_equals_two_launches(moe, oracle, dev, dtype, E, H, I, T, K, act):
+    """Blocks of 256 with 16-bit dtypes enqueue the gate-up and the down pass as one
+    launch, the down tiles of an m-block starting once its gate-up tiles are counted
+    in.  Same tiles, same arithmetic: the result equals that of two launches bit for
+    bit, on every repetition (a down tile that started early would read stale rows)."""
+    fm = moe.fused_moe
+    x, w13, w2, logits = _layer(E, H, I, T, K, 300 + E, dtype)
+    tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
+    d = lambda t: t.to(dev)
+    x, w13, w2, tw, ids = d(x), d(w13), d(w2), d(tw), d(ids)
+    so, eo, npp = fm.moe_align_block_size(ids, 256, E)
+    two = torch.empty_like(x)
+    fm.launch_fused_experts(x, two, w13, w2, None, None, None, None, tw, so, eo, npp, 256, activation=act,
+                            passes=7 | 8)
+    _close(two, oracle.fused_experts_ref(x.cpu(), w13.cpu(), w2.cpu(), tw.cpu(), ids.cpu(), activation=act))
+    ws = None
+    for rep in range(6):
+        one = torch.full_like(x, float("nan"))
+        # a fresh workspace each time: the counters and the intermediate start from whatever memory holds
+        fm.launch_fused_experts(x, one, w13, w2, None, None, None, None, tw, so, eo, npp, 256, activation=act)
+        torch.cuda.synchronize()
+        assert torch.equal(one, two), f"repetition {rep}: {(one != two).sum().item()} elements differ"

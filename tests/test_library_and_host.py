@@ -66,7 +66,9 @@ def test_argument_validation_without_gpu(moe):
     want = 0
     for rows, cols in ((67584 + 128 * 127, 768), (67584, 2048)):
         want += -(-rows * cols * 2 // 256) * 256
-    assert L.moe_fused_experts_workspace_bytes(8448, 2048, 768, 128, 8, 128, 2, 2) == want + 256  # + XCD range table
+    # + one counter per 256-slot block (one-launch form of the large-tile passes) + XCD range table
+    counters = -(-(-(-(67584 + 128 * 127) // 256) * 4) // 256) * 256
+    assert L.moe_fused_experts_workspace_bytes(8448, 2048, 768, 128, 8, 128, 2, 2) == want + counters + 256
     # act dtype code 2 = bf16: streaming blocks, then the large tile from 48 rows per expert on
     for m, bm in ((256, 32), (512, 64), (768, 256), (8448, 256)):
         assert L.moe_preferred_block_size(m, 128, 8, 2, 2) == bm
