@@ -1614,7 +1614,6 @@ int elem_size(int dtype) { return dtype == MOE_F32 ? 4 : (dtype == MOE_E4M3 ? 1 
 }  // namespace
 
 MOE_EXPORT int moe_preferred_block_size(int M, int E, int K, int act_dtype, int weight_dtype) {
-  (void)weight_dtype;
   if (E < 1) return 64;
   const int64_t avg = static_cast<int64_t>(M) * K / E;  // routed rows per expert
   if (act_dtype == MOE_F32) {  // register-staged kernels only: the M tile follows the load
@@ -1623,12 +1622,14 @@ MOE_EXPORT int moe_preferred_block_size(int M, int E, int K, int act_dtype, int 
     if (avg >= 24) return 64;
     return 32;
   }
-  // 16-bit activations: the large-tile kernel streams weights so much better than the
-  // register-staged ones that it wins from about 48 rows per expert on, padding included
-  // (Qwen3-30B-A3B layer, 768 tokens: 0.27 ms against 0.30 ms with blocks of 64; 3072
-  // tokens: 0.48 ms against 0.62 ms); below that the streaming kernel's 32-slot blocks.
-  if (avg >= 48) return 256;
-  if (avg >= 24) return 64;
+  // 16-bit activations: the large-tile kernel, whose two passes go out as one launch,
+  // or the streaming kernel with 32-slot blocks.  Padding fragments of a 256-slot block
+  // cost neither loads nor MFMAs, so the large tile wins from 16 routed rows per expert
+  // on (Qwen3-30B-A3B layer: 0.171 against 0.184 ms at 256 tokens, 0.210 against 0.235 ms
+  // at 512; at 192 tokens the streaming kernel still leads, 0.171 against 0.189 ms).
+  // e4m3 weights quantise the intermediate between the passes (two launches): from 32
+  // rows per expert on (0.181 against 0.193 ms at 512 tokens; 0.172 against 0.166 at 384).
+  if (avg >= (weight_dtype == MOE_E4M3 ? 32 : 16)) return 256;
   return 32;
 }
 

@@ -69,9 +69,12 @@ def test_argument_validation_without_gpu(moe):
     # + one counter per 256-slot block (one-launch form of the large-tile passes) + XCD range table
     counters = -(-(-(-(67584 + 128 * 127) // 256) * 4) // 256) * 256
     assert L.moe_fused_experts_workspace_bytes(8448, 2048, 768, 128, 8, 128, 2, 2) == want + counters + 256
-    # act dtype code 2 = bf16: streaming blocks, then the large tile from 48 rows per expert on
-    for m, bm in ((256, 32), (512, 64), (768, 256), (8448, 256)):
+    # act dtype code 2 = bf16: streaming blocks, then the large tile from 16 rows per expert on
+    for m, bm in ((64, 32), (192, 32), (256, 256), (512, 256), (768, 256), (8448, 256)):
         assert L.moe_preferred_block_size(m, 128, 8, 2, 2) == bm
+    # e4m3 weights (code 3) quantise the intermediate between the passes: from 32 rows per expert on
+    for m, bm in ((256, 32), (384, 32), (512, 256), (8448, 256)):
+        assert L.moe_preferred_block_size(m, 128, 8, 2, 3) == bm
     # fp32 (code 0) has no large-tile kernel: the M tile follows the load
     for m, bm in ((256, 32), (768, 64), (2048, 128), (8448, 256)):
         assert L.moe_preferred_block_size(m, 128, 8, 0, 0) == bm
