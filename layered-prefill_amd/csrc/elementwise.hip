@@ -94,8 +94,17 @@ __device__ __forceinline__ uint8_t f32_to_e4m3(float v) {
   return static_cast<uint8_t>(__builtin_amdgcn_cvt_pk_fp8_f32(v, v, 0, false) & 0xff);
 }
 
+// Two values at once: bits 0-7 the code of a, bits 8-15 the code of b.
+__device__ __forceinline__ uint32_t f32x2_to_e4m3(float a, float b) {
+  a = __builtin_amdgcn_fmed3f(a, -448.f, 448.f);
+  b = __builtin_amdgcn_fmed3f(b, -448.f, 448.f);
+  return static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false)) & 0xffffu;
+}
+
 // One wavefront per row: s = amax|row| / 448 (1 for an all-zero row),
-// q = e4m3(row / s).
+// q = e4m3(row * (1 / s)): one correctly rounded division per row, then one
+// multiplication per element (a division per element made the kernel
+// VALU-bound: 48 us for 67584 x 768 against 28 us of memory time).
 template <typename El>
 __global__ __launch_bounds__(kThreads) void quant_rows_e4m3_kernel(
     const typename El::S* __restrict__ w, int64_t rows, int cols, uint8_t* __restrict__ q,
@@ -111,7 +120,8 @@ __global__ __launch_bounds__(kThreads) void quant_rows_e4m3_kernel(
   for (int m = 32; m > 0; m /= 2) amax = fmaxf(amax, __shfl_xor(amax, m, kWave));
   const float s = amax > 0.f ? amax / 448.f : 1.f;
   if (lane == 0) scales[row] = s;
-  for (int c = lane; c < cols; c += kWave) q[row * cols + c] = f32_to_e4m3(El::ld(src[c]) / s);
+  const float inv = 1.0f / s;
+  for (int c = lane; c < cols; c += kWave) q[row * cols + c] = f32_to_e4m3(El::ld(src[c]) * inv);
 }
 
 // 16-bit sources with up to NV * 512 columns: the row stays in registers between
@@ -144,6 +154,7 @@ __global__ __launch_bounds__(kThreads) void quant_rows_e4m3_vec_kernel(
   for (int m = 32; m > 0; m /= 2) amax = fmaxf(amax, __shfl_xor(amax, m, kWave));
   const float s = amax > 0.f ? amax / 448.f : 1.f;
   if (lane == 0) scales[row] = s;
+  const float inv = 1.0f / s;
   uint2* dst = reinterpret_cast<uint2*>(q + row * cols);
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -152,11 +163,10 @@ __global__ __launch_bounds__(kThreads) void quant_rows_e4m3_vec_kernel(
     const uint32_t wds[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
     uint32_t o[2] = {0, 0};
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint32_t lo = f32_to_e4m3(El::ld(static_cast<uint16_t>(wds[j])) / s);
-      const uint32_t hi = f32_to_e4m3(El::ld(static_cast<uint16_t>(wds[j] >> 16)) / s);
-      o[j >> 1] |= (lo | (hi << 8)) << (16 * (j & 1));
-    }
+    for (int j = 0; j < 4; ++j)
+      o[j >> 1] |= f32x2_to_e4m3(El::ld(static_cast<uint16_t>(wds[j])) * inv,
+                                 El::ld(static_cast<uint16_t>(wds[j] >> 16)) * inv)
+                   << (16 * (j & 1));
     dst[c] = uint2{o[0], o[1]};
   }
 }

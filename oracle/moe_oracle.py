@@ -222,20 +222,23 @@ def dequant_e4m3(code: torch.Tensor) -> torch.Tensor:
 
 def quant_weight_per_channel(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """[E, N, K] -> (codes uint8 [E,N,K], scales f32 [E,N]) with
-    s[e,n] = amax_k |w[e,n,k]| / 448 (1.0 for an all-zero channel)."""
+    s[e,n] = amax_k |w[e,n,k]| / 448 (1.0 for an all-zero channel) and codes
+    e4m3(w * (1 / s)), every operation a rounded fp32 one (the reciprocal form
+    of dynamic fp8 quantisers: one division per row, one product per element)."""
     wf = _cpu(w).float()
     amax = wf.abs().amax(dim=-1)
     s = torch.where(amax > 0, amax / E4M3_MAX, torch.ones_like(amax))
-    q = quant_e4m3(wf / s[..., None])
+    q = quant_e4m3(wf * (1.0 / s)[..., None])
     return q, s
 
 
 def quant_act_per_token(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    """[R, K] -> (codes uint8, scales f32 [R]) with s[r] = amax|x[r]| / 448."""
+    """[R, K] -> (codes uint8, scales f32 [R]) with s[r] = amax|x[r]| / 448 and
+    codes e4m3(x * (1 / s)), as ``quant_weight_per_channel``."""
     xf = _cpu(x).float()
     amax = xf.abs().amax(dim=-1)
     s = torch.where(amax > 0, amax / E4M3_MAX, torch.ones_like(amax))
-    q = quant_e4m3(xf / s[:, None])
+    q = quant_e4m3(xf * (1.0 / s)[:, None])
     return q, s
 
 

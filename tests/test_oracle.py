@@ -271,6 +271,14 @@ def test_per_channel_and_per_token_scales(oracle):
     assert torch.allclose(s, w.abs().amax(-1) / 448)
     deq = oracle.dequant_e4m3(q) * s[..., None]
     assert ((deq - w).abs() <= w.abs().amax(-1, keepdim=True) * 2 ** -4 + 1e-9).all()
+    # the largest element of every channel lands on the largest code, and the per-token
+    # quantiser is the same function of a row
+    assert (oracle.dequant_e4m3(q).abs().amax(-1) == 448).all()
+    q0, s0 = oracle.quant_act_per_token(w[0])
+    assert torch.equal(q0, q[0]) and torch.equal(s0, s[0])
+    # codes are those of the fp32 product with the rounded reciprocal of the scale
+    want = oracle.quant_e4m3(w[1] * (torch.tensor(1.0) / s[1])[:, None])
+    assert torch.equal(q[1], want)
 
 
 # ----------------------------------------------------------------- expert MLP
