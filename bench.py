@@ -244,15 +244,24 @@ def trace_mix(moe, layer: Layer, steps: int):
             "layer_tokens_per_s": round(t_tok / (t_ms * 1e-3), 0)}
 
 
-def time_stages(layer: Layer, steps: int):
+def time_stages(layer: Layer, steps: int, warmup: int = 10):
+    """Per-stage times from events recorded inside a run of back-to-back steps: no
+    synchronisation between steps, so the GPU is in the same sustained state as in
+    the timed loop (after an idle gap the first ~20 steps of this layer run up to
+    15 % slower while the power management settles)."""
     names = ["topk_softmax", "moe_align_block_size", "gate_up_gemm_act", "down_gemm_weighted",
              "topk_combine"]
     per = {n: [] for n in names + ["both_gemm_passes"]}
     ids = None
+    for _ in range(warmup):
+        layer.step_instrumented(_events(8))
+    evs = []
     for _ in range(steps):
         ev = _events(8)
         ids = layer.step_instrumented(ev)
-        torch.cuda.synchronize()
+        evs.append(ev)
+    torch.cuda.synchronize()
+    for ev in evs:
         for i, n in enumerate(names):
             per[n].append(ev[i].elapsed_time(ev[i + 1]))
         per["both_gemm_passes"].append(ev[6].elapsed_time(ev[7]))
@@ -336,8 +345,10 @@ def cpu_baseline(moe, name: str, runs: int):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=5)
+    # defaults long enough to measure the sustained rate: after an idle gap the first
+    # ~20 steps (20 ms) of this layer run up to 15 % slower while the clocks settle
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="layered_8192p_256d",
                     choices=["layered_8192p_256d", "decode_256"])
     ap.add_argument("--no-cpu-baseline", action="store_true")

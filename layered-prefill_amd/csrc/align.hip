@@ -11,8 +11,10 @@
 // which is the stable order and needs no global atomics.
 //
 // Small inputs run as ONE workgroup of 16 wavefronts (histogram, scans and
-// scatter in LDS); larger ones as three launches (count / scan / scatter)
-// with the per-segment histograms in the caller's workspace.
+// scatter in LDS); larger ones as two launches (count, then scan + scatter with
+// every workgroup deriving its own prefixes) with the per-segment histograms in
+// the caller's workspace; three launches (count / scan / scatter) when the
+// tables of the second launch would not fit in LDS.
 #include "common.h"
 
 namespace {
@@ -256,6 +258,105 @@ __global__ __launch_bounds__(kScanThreads) void align_scan_kernel(
                            expert_cap, num_post_pad);
 }
 
+// Scan and scatter in one launch: every workgroup owns kScanWaves consecutive
+// segments and derives what it needs from the per-segment histograms by itself
+// (they are a few tens of KB and sit in L2): the totals per expert, the counts
+// in front of its own segments, the padded prefix over experts.  Then each of
+// its wavefronts scatters one segment, and the workgroups share the padding and
+// expert_ids writes.  No workgroup waits for another.
+// LDS: part[nwg][E] | own[kScanWaves][E] | cum[E+1] | tot[E] | wave_tot[kScanWaves+1]
+__global__ __launch_bounds__(kScanThreads) void align_place_kernel(
+    const void* __restrict__ ids, int dtype, int64_t numel, int E, int BM, int id_bits,
+    const int32_t* __restrict__ seg_cnt, int nseg, int32_t* __restrict__ sorted_ids,
+    int64_t sorted_cap, int32_t* __restrict__ expert_ids, int64_t expert_cap,
+    int32_t* __restrict__ num_post_pad) {
+  extern __shared__ int lds[];
+  const int nwg = gridDim.x;
+  volatile int* part = lds;
+  volatile int* own = lds + nwg * E;
+  volatile int* cum = own + kScanWaves * E;
+  volatile int* tot = cum + (E + 1);
+  volatile int* wave_tot = tot + E;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  // thread t sums expert t % E over the segments of workgroups t / E, t / E + R, ...
+  // (a wavefront reads 64 consecutive experts of one segment: one 256-byte line)
+  const int R = kScanThreads / E;
+  const int e = threadIdx.x % E, r = threadIdx.x / E;
+  if (r < R) {
+    for (int q = r; q < nwg; q += R) {
+      const int s0 = q * kScanWaves;
+      int c[kScanWaves];
+#pragma unroll
+      for (int i = 0; i < kScanWaves; ++i)
+        c[i] = s0 + i < nseg ? seg_cnt[static_cast<size_t>(s0 + i) * E + e] : 0;
+      int sum = 0;
+#pragma unroll
+      for (int i = 0; i < kScanWaves; ++i) sum += c[i];
+      part[q * E + e] = sum;
+      if (q == static_cast<int>(blockIdx.x)) {
+#pragma unroll
+        for (int i = 0; i < kScanWaves; ++i) own[i * E + e] = c[i];
+      }
+    }
+  }
+  __syncthreads();
+  int padded = 0;
+  if (threadIdx.x < E) {
+    int before = 0, total = 0;
+    for (int q = 0; q < nwg; ++q) {
+      const int v = part[q * E + threadIdx.x];
+      if (q < static_cast<int>(blockIdx.x)) before += v;
+      total += v;
+    }
+    tot[threadIdx.x] = total;
+    padded = (total + BM - 1) / BM * BM;
+    // own[w][e] becomes the number of ids of expert e in front of segment w of this workgroup
+    int running = before;
+    for (int w = 0; w < kScanWaves; ++w) {
+      const int c = own[w * E + threadIdx.x];
+      own[w * E + threadIdx.x] = running;
+      running += c;
+    }
+  }
+  const int excl = block_exclusive_scan(padded, wave_tot);
+  if (threadIdx.x < E) cum[threadIdx.x] = excl;
+  if (threadIdx.x == E) cum[E] = excl;  // E < kScanThreads: threads past E add 0
+  if (E == kScanThreads && threadIdx.x == 0) cum[E] = wave_tot[kScanWaves];
+  __syncthreads();
+  // this workgroup's share of expert_ids, of the padding inside the experts' last
+  // blocks and of the tail behind the padded total
+  const int total = cum[E];
+  if (blockIdx.x == 0 && threadIdx.x == 0) *num_post_pad = total;
+  const int used_blocks = total / BM;
+  const int64_t gtid = static_cast<int64_t>(blockIdx.x) * kScanThreads + threadIdx.x;
+  const int64_t gthreads = static_cast<int64_t>(nwg) * kScanThreads;
+  for (int64_t b = gtid; b < expert_cap; b += gthreads) {
+    int owner = 0;
+    if (b < used_blocks) {
+      const int pos = static_cast<int>(b) * BM;
+      int lo = 1, hi = E;  // first j in [1, E] with cum[j] > pos; the block belongs to expert j - 1
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (cum[mid] > pos) hi = mid; else lo = mid + 1;
+      }
+      owner = lo - 1;
+    }
+    expert_ids[b] = owner;
+  }
+  for (int x = blockIdx.x * kScanWaves + wave; x < E; x += nwg * kScanWaves) {
+    const int beg = cum[x] + tot[x], end = cum[x + 1];
+    for (int p = beg + lane; p < end; p += kWave) sorted_ids[p] = static_cast<int32_t>(numel);
+  }
+  for (int64_t p = total + gtid; p < sorted_cap; p += gthreads) sorted_ids[p] = static_cast<int32_t>(numel);
+  // per-wavefront running slots: ids in front of the segment + expert base
+  const int sg = blockIdx.x * kScanWaves + wave;
+  if (sg >= nseg) return;
+  for (int x = lane; x < E; x += kWave) own[wave * E + x] += cum[x];
+  const int64_t beg = static_cast<int64_t>(sg) * kSegLen;
+  const int64_t end = beg + kSegLen < numel ? beg + kSegLen : numel;
+  scatter_segment(ids, dtype, beg, end, E, id_bits, own + wave * E, sorted_ids);
+}
+
 __global__ __launch_bounds__(kWave) void align_scatter_kernel(
     const void* __restrict__ ids, int dtype, int64_t numel, int E, int id_bits,
     const int32_t* __restrict__ seg_base, const int32_t* __restrict__ cum,
@@ -327,6 +428,15 @@ MOE_EXPORT int moe_align_block_size(const void* topk_ids, int ids_dtype, int64_t
   int32_t* cum = seg_cnt + static_cast<size_t>(nseg) * E;
   hipLaunchKernelGGL(align_count_kernel, dim3(nseg), dim3(kWave), E * sizeof(int), s, topk_ids,
                      ids_dtype, numel, E, seg_cnt);
+  // scan and scatter as one launch while its LDS tables fit
+  const int nwg = (nseg + kScanWaves - 1) / kScanWaves;
+  const size_t place_lds = (static_cast<size_t>(nwg + kScanWaves) * E + (E + 1) + E + kScanWaves + 1) * sizeof(int);
+  if (place_lds <= 60 * 1024) {
+    hipLaunchKernelGGL(align_place_kernel, dim3(nwg), dim3(kScanThreads), place_lds, s, topk_ids, ids_dtype,
+                       numel, E, block_size, id_bits, seg_cnt, nseg, sorted_token_ids, sorted_cap,
+                       expert_ids, expert_cap, num_tokens_post_pad);
+    return moe_check_launch("moe_align_block_size (count + place)");
+  }
   hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, seg_cnt, nseg, E,
                      block_size, static_cast<int>(numel), cum, sorted_token_ids, sorted_cap,
                      expert_ids, expert_cap, num_tokens_post_pad);

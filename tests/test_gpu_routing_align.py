@@ -82,6 +82,7 @@ ALIGN_CASES = [
     (2048, 128, 64), (2048, 128, 128), (6144, 128, 64), (16384, 128, 32), (16385, 128, 32),
     (67584, 128, 64), (67584, 128, 128), (67584, 128, 16), (524288, 128, 128), (30000, 60, 7),
     (5000, 1000, 16), (70000, 1024, 8), (3000, 600, 32), (40000, 512, 64), (1000, 2, 256),
+    (67584, 128, 256), (100000, 96, 256), (16900, 3, 32), (200000, 256, 64),
 ]
 
 
