@@ -117,10 +117,7 @@ __device__ __forceinline__ void scatter_segment(const void* ids, int dtype, int6
                                                 int64_t end, int E, int id_bits,
                                                 volatile int* run, int32_t* sorted_ids) {
   const int lane = threadIdx.x % kWave;
-  for (int64_t base = beg; base < end; base += kWave) {
-    const int64_t i = base + lane;
-    int id = -1;
-    if (i < end) id = load_id(ids, dtype, i);
+  auto place = [&](int64_t i, int id) {
     const bool valid = id >= 0 && id < E;
     const uint64_t grp = same_id_lanes(id, valid, id_bits);
     if (valid) {
@@ -129,6 +126,20 @@ __device__ __forceinline__ void scatter_segment(const void* ids, int dtype, int6
       sorted_ids[slot] = static_cast<int32_t>(i);
       if (below == 0) run[id] = slot + __popcll(grp);
     }
+  };
+  // the ids of up to eight steps are fetched at once: loaded step by step, every
+  // step would wait out one memory latency before its ballots
+  constexpr int PF = 8;
+  for (int64_t base = beg; base < end; base += PF * kWave) {
+    int id[PF];
+#pragma unroll
+    for (int j = 0; j < PF; ++j) {
+      const int64_t i = base + j * kWave + lane;
+      id[j] = i < end ? load_id(ids, dtype, i) : -1;
+    }
+#pragma unroll
+    for (int j = 0; j < PF; ++j)
+      if (base + j * kWave < end) place(base + j * kWave + lane, id[j]);
   }
 }
 
@@ -187,10 +198,15 @@ __global__ __launch_bounds__(kWave) void align_count_kernel(const void* __restri
   __syncthreads();
   const int64_t beg = static_cast<int64_t>(blockIdx.x) * kSegLen;
   const int64_t end = beg + kSegLen < numel ? beg + kSegLen : numel;
-  for (int64_t i = beg + lane; i < end; i += kWave) {
-    const int id = load_id(ids, dtype, i);
-    if (id >= 0 && id < E) atomicAdd(&lds[id], 1);
+  int id[kSegLen / kWave];  // all loads of the segment in flight together
+#pragma unroll
+  for (int j = 0; j < kSegLen / kWave; ++j) {
+    const int64_t i = beg + j * kWave + lane;
+    id[j] = i < end ? load_id(ids, dtype, i) : -1;
   }
+#pragma unroll
+  for (int j = 0; j < kSegLen / kWave; ++j)
+    if (id[j] >= 0 && id[j] < E) atomicAdd(&lds[id[j]], 1);
   __syncthreads();
   for (int e = lane; e < E; e += kWave) seg_cnt[static_cast<size_t>(blockIdx.x) * E + e] = lds[e];
 }
