@@ -31,10 +31,11 @@ METRIC = "MoE layer TFLOP/s @8192+256 tok & decode HBM GB/s, Qwen3-30B-A3B layer
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs (profiles/hbm_traffic_gate_up_kernels.txt): fetch + write bytes.
-MEASURED_TRAFFIC_BYTES = {"layered_8192p_256d": 1773152256 + 114690048,
-                          "decode_256": 571137843 + 3340083}
+# HBM bytes per launch of the dominant kernel (both grouped GEMMs in one launch), from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (profiles/hbm_traffic_grouped_gemm_kernels.txt): fetch + write bytes.
+MEASURED_TRAFFIC_BYTES = {"layered_8192p_256d": 2528221184 + 386402304,
+                          "decode_256": 763348992 + 11639808}
 
 
 def _events(n):
@@ -224,7 +225,8 @@ def trace_mix(moe, layer: Layer, steps: int):
             tw, ids, _ = moe.fused_topk(x, logits, s.top_k, True)
             return moe.fused_experts(x, layer.w13, layer.w2, None, None, tw, ids)
 
-        for _ in range(3):
+        # sustained rate per bucket: about 40 ms of warm-up, then `steps` timed calls
+        for _ in range(max(3, min(200, int(40.0 / (0.1 + b * 1e-4))))):
             step()
         ev = _events(2)
         ev[0].record()
@@ -452,7 +454,7 @@ def main() -> int:
 
     out["router_gate"] = time_router_gate(moe, main_layer, 50)
     if compute_bound and not a.no_trace_mix:
-        out["trace_mix"] = trace_mix(moe, main_layer, 10)
+        out["trace_mix"] = trace_mix(moe, main_layer, max(10, a.steps // 4))
     if compute_bound and a.chunk_mode != "off":
         out["chunk_amplification"] = chunk_amplification(moe, main_layer, max(2, a.steps // 10), a.chunk_mode)
     if compute_bound and not a.no_fp8:
