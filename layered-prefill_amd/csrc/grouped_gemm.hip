@@ -1150,8 +1150,10 @@ __global__ __launch_bounds__(kThreads, 1) void big_fused_kernel(const GemmParams
 
 // Cuts the live m-blocks of a large-tile launch into one contiguous range per XCD
 // with equal estimated work instead of equal counts.  A block of an expert that
-// received at most 32 (64) rows is weight streaming only and costs about 0.53
-// (0.69) of a full one; with equal counts the XCDs finished up to 25 % apart.
+// received at most 32 (64) rows is weight streaming only and costs about 0.56
+// (0.70) of a full one, a partly filled one 0.97 (its six gate-up and eight down
+// tiles: 318 / 394 / 542 / 562 us of CU time at 8448 tokens); with equal counts
+// the XCDs finished up to 25 % apart.
 // Ranges stay contiguous so that the blocks of one expert keep sharing its
 // weights through one L2.  No range is longer than cap_mb blocks (the grid has
 // that many slots per XCD).  One workgroup; bounds[0..8] in m-blocks.
@@ -1169,7 +1171,7 @@ __global__ __launch_bounds__(kPlanThreads) void big_plan_kernel(const int32_t* _
   auto weight = [&](int mb) {
     if (mb >= live_mb) return 0;
     const int32_t* s = sorted_ids + static_cast<int64_t>(mb) * kBigBM;
-    return s[32] >= numel ? 17 : (s[64] >= numel ? 22 : 32);
+    return s[32] >= numel ? 36 : (s[64] >= numel ? 45 : (s[kBigBM - 1] >= numel ? 62 : 64));
   };
   // inclusive scan of `v` over the workgroup, plus the workgroup total
   auto scan = [&](int v, int& total) {
