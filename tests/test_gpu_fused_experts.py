@@ -462,3 +462,29 @@ def test_one_launch_form_equals_two_launches(moe, oracle, dev, dtype, E, H, I, T
         fm.launch_fused_experts(x, one, w13, w2, None, None, None, None, tw, so, eo, npp, 256, activation=act)
         torch.cuda.synchronize()
         assert torch.equal(one, two), f"repetition {rep}: {(one != two).sum().item()} elements differ"
+
+
+@pytest.mark.gpu
+def test_empty_batch_and_chunk_boundary(moe, oracle, dev):
+    """No tokens: empty results, nothing enqueued.  More than 65536 tokens: the
+    host loop of nanovllm/layers/for_moe/fused_moe.py:503,547-566 runs the path in
+    chunks of 65536 rows, the last one ragged with its own block size."""
+    E, H, I, K = 8, 64, 64, 2
+    g = torch.Generator().manual_seed(12)
+    w13 = (torch.randn(E, 2 * I, H, generator=g) * 0.05).bfloat16()
+    w2 = (torch.randn(E, H, I, generator=g) * 0.05).bfloat16()
+    d = lambda t: t.to(dev)
+    x0 = torch.empty(0, H, dtype=torch.bfloat16, device=dev)
+    tw0, ids0, tei0 = moe.fused_topk(x0, torch.empty(0, E, device=dev), K, True)
+    assert tuple(tw0.shape) == (0, K) and tuple(ids0.shape) == (0, K) and tuple(tei0.shape) == (0, K)
+    out0 = moe.fused_experts(x0, d(w13), d(w2), None, None, tw0, ids0)
+    assert tuple(out0.shape) == (0, H) and out0.dtype == torch.bfloat16
+    T = 65536 + 300
+    x = torch.randn(T, H, generator=g).bfloat16()
+    logits = torch.randn(T, E, generator=g)
+    tw, ids, _ = moe.fused_topk(d(x), d(logits), K, True)
+    out = moe.fused_experts(d(x), d(w13), d(w2), None, None, tw, ids)
+    torch.cuda.synchronize()
+    rows = torch.cat([torch.arange(0, 65536, 4099), torch.arange(65536 - 3, T, 7)])
+    ref = oracle.fused_experts_ref(x[rows], w13, w2, tw.cpu()[rows], ids.cpu()[rows])
+    _close(out[rows.to(dev)], ref)
