@@ -488,3 +488,35 @@ def test_empty_batch_and_chunk_boundary(moe, oracle, dev):
     rows = torch.cat([torch.arange(0, 65536, 4099), torch.arange(65536 - 3, T, 7)])
     ref = oracle.fused_experts_ref(x[rows], w13, w2, tw.cpu()[rows], ids.cpu()[rows])
     _close(out[rows.to(dev)], ref)
+
+
+@pytest.mark.gpu
+def test_one_launch_form_on_two_streams(moe, oracle, dev):
+    """Two layers enqueued side by side on two streams, each with its own workspace:
+    the one-launch kernels of both share the CUs, and a down tile only ever waits for
+    gate-up tiles of its own launch that were started before it.  Results equal the
+    ones computed alone, bit for bit."""
+    fm = moe.fused_moe
+    d = lambda t: t.to(dev)
+    jobs = []
+    for E, H, I, T, K, seed in ((16, 512, 256, 2500, 4, 71), (64, 256, 128, 6000, 8, 72)):
+        x, w13, w2, logits = _layer(E, H, I, T, K, seed, torch.bfloat16)
+        tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
+        x, w13, w2, tw, ids = d(x), d(w13), d(w2), d(tw), d(ids)
+        so, eo, npp = fm.moe_align_block_size(ids, 256, E)
+        ws = torch.empty(moe._lib.lib().moe_fused_experts_workspace_bytes(
+            T, H, I, E, K, 256, moe._lib.DTYPE_CODE[torch.bfloat16], moe._lib.DTYPE_CODE[torch.bfloat16]),
+            dtype=torch.uint8, device=dev)
+        alone = torch.empty_like(x)
+        fm.launch_fused_experts(x, alone, w13, w2, None, None, None, None, tw, so, eo, npp, 256, workspace=ws)
+        jobs.append(dict(x=x, w13=w13, w2=w2, tw=tw, so=so, eo=eo, npp=npp, ws=ws, alone=alone,
+                         out=torch.empty_like(x), stream=torch.cuda.Stream(device=dev)))
+    torch.cuda.synchronize()
+    for rep in range(8):
+        for j in jobs:
+            with torch.cuda.stream(j["stream"]):
+                fm.launch_fused_experts(j["x"], j["out"], j["w13"], j["w2"], None, None, None, None, j["tw"],
+                                        j["so"], j["eo"], j["npp"], 256, workspace=j["ws"])
+    torch.cuda.synchronize()
+    for j in jobs:
+        assert torch.equal(j["out"], j["alone"])
