@@ -126,7 +126,8 @@ typedef struct MoeFusedExpertsArgs {
   const int32_t* sorted_token_ids;    /* from moe_align_block_size                  */
   const int32_t* expert_ids;
   const int32_t* num_tokens_post_pad; /* read on the device only                    */
-  void* workspace;
+  void* workspace;           /* intermediates and launch bookkeeping of this call: one call at a
+                                time per workspace (two calls in flight need two workspaces) */
   int64_t workspace_bytes;
   /* element strides of the expert dimension and the row dimension of the
      weights (last dimension is contiguous) */
