@@ -84,6 +84,22 @@ int moe_align_block_size(const void* topk_ids, int ids_dtype, int64_t numel, int
                          int32_t* expert_ids, int64_t expert_cap, int32_t* num_tokens_post_pad,
                          void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The same alignment for block_size 256, which also leaves in the workspace of the
+ * moe_fused_experts call that follows what that call would otherwise compute with a launch
+ * of its own: the per-XCD m-block ranges of the large-tile kernel (`plan_bounds`, 9 int32)
+ * and its cleared per-block counters (`plan_done`, `plan_num_done` int32); the four values
+ * come from moe_fused_experts_plan_layout, and that call is then made with bit 16 of
+ * `passes` set.  No counterpart in the reference (its Triton launch needs no plan).
+ * moe_align_can_plan says whether the size is served (tables of E x segments in LDS). */
+int moe_align_can_plan(int64_t numel, int E);
+int moe_align_block_size_planned(const void* topk_ids, int ids_dtype, int64_t numel, int E,
+                                 int block_size, int32_t* sorted_token_ids, int64_t sorted_cap,
+                                 int32_t* expert_ids, int64_t expert_cap,
+                                 int32_t* num_tokens_post_pad, void* workspace,
+                                 int64_t workspace_bytes, void* stream, int32_t* plan_bounds,
+                                 int32_t* plan_done, int plan_num_done, int plan_cap_mb);
+
+
 /* Replaces `silu_and_mul` (csrc/activation_kernels.cu:68-87, bound at
  * csrc/ops.cpp:29-31,99-103): out[r,i] = T(silu(in[r,i])) * in[r,d+i]. */
 int moe_silu_and_mul(void* out, const void* in, int64_t rows, int d, int dtype, void* stream);
@@ -145,7 +161,8 @@ typedef struct MoeFusedExpertsArgs {
      times routed weight, 4 top-k combine; 0 means all three.  Lets a profiler
      or benchmark time one pass alone (the later passes then read whatever the
      workspace holds).  Bit 8 keeps the two GEMM passes in separate launches
-     where the library would otherwise enqueue them as one. */
+     where the library would otherwise enqueue them as one.  Bit 16: the
+     workspace already holds the plan (moe_align_block_size_planned). */
   int32_t passes;
   void* stream;
 } MoeFusedExpertsArgs;
@@ -153,6 +170,11 @@ typedef struct MoeFusedExpertsArgs {
 int64_t moe_fused_experts_workspace_bytes(int T, int H, int I, int E, int K, int block_size,
                                           int act_dtype, int weight_dtype);
 int moe_fused_experts(const MoeFusedExpertsArgs* args);
+/* Offsets into the workspace (and sizes) of the plan that moe_align_block_size_planned
+ * writes for a moe_fused_experts call of these sizes; returns 1 when the call uses one. */
+int moe_fused_experts_plan_layout(int T, int H, int I, int E, int K, int block_size, int act_dtype,
+                                  int weight_dtype, int64_t* bounds_offset, int64_t* done_offset,
+                                  int32_t* num_done, int32_t* cap_mb);
 
 /* The M-tile (alignment block_size) the grouped GEMMs run best with for M
  * tokens; plays the role of config["BLOCK_SIZE_M"] chosen by

@@ -27,6 +27,7 @@ EXPORTS = (
     "moe_align_block_size", "moe_silu_and_mul", "moe_swigluoai_and_mul", "moe_sum",
     "moe_fused_experts_workspace_bytes", "moe_fused_experts", "moe_preferred_block_size",
     "moe_quant_rows_e4m3", "moe_gate_topk_softmax", "moe_add_rms_norm",
+    "moe_align_can_plan", "moe_align_block_size_planned", "moe_fused_experts_plan_layout",
 )
 
 
@@ -74,6 +75,13 @@ def _declare(L: ctypes.CDLL) -> None:
     L.moe_align_workspace_bytes.argtypes = [i64, i32]
     L.moe_align_block_size.restype = i32
     L.moe_align_block_size.argtypes = [p, i32, i64, i32, i32, p, i64, p, i64, p, p, i64, p]
+    L.moe_align_can_plan.restype = i32
+    L.moe_align_can_plan.argtypes = [i64, i32]
+    L.moe_align_block_size_planned.restype = i32
+    L.moe_align_block_size_planned.argtypes = [p, i32, i64, i32, i32, p, i64, p, i64, p, p, i64, p, p, p, i32, i32]
+    L.moe_fused_experts_plan_layout.restype = i32
+    L.moe_fused_experts_plan_layout.argtypes = [i32] * 8 + [ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
+                                                            ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)]
     L.moe_silu_and_mul.restype = i32
     L.moe_silu_and_mul.argtypes = [p, p, i64, i32, i32, p]
     L.moe_swigluoai_and_mul.restype = i32

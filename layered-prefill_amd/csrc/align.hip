@@ -143,10 +143,57 @@ __device__ __forceinline__ void scatter_segment(const void* ids, int dtype, int6
   }
 }
 
+// What big_plan_kernel (grouped_gemm.hip) derives from the aligned ids, derived from the
+// per-expert counts instead, for an alignment with blocks of 256 slots: the m-block
+// ranges [bounds[x], bounds[x+1]) of the 8 XCDs with equal estimated work (a block costs
+// 36 / 45 / 62 / 64 with at most 32 / at most 64 / fewer than 256 / 256 real slots), no range
+// longer than cap_mb, and the per-block counters of the one-launch form cleared.  Saves the
+// large-tile path a launch.  Called by all kScanThreads threads; contains barriers.
+constexpr int kPlanBlock = 256, kPlanXcds = 8;
+__device__ void plan_from_counts(const volatile int* cum, const volatile int* tot, int E, int cap_mb,
+                                 int32_t* bounds, int32_t* done, int num_done, volatile int* wave_tot) {
+  __shared__ int s_b[kPlanXcds + 1];
+  for (int i = threadIdx.x; i < num_done; i += kScanThreads) done[i] = 0;
+  const int live_mb = cum[E] / kPlanBlock;
+  int w = 0, nb = 0, first = 0;
+  if (static_cast<int>(threadIdx.x) < E) {
+    nb = (cum[threadIdx.x + 1] - cum[threadIdx.x]) / kPlanBlock;
+    first = cum[threadIdx.x] / kPlanBlock;
+    if (nb > 0) {
+      const int r = tot[threadIdx.x] - (nb - 1) * kPlanBlock;  // real slots of the expert's last block
+      w = (nb - 1) * 64 + (r <= 32 ? 36 : (r <= 64 ? 45 : (r < kPlanBlock ? 62 : 64)));
+    }
+  }
+  const int excl = block_exclusive_scan(w, wave_tot);
+  const int total = wave_tot[kScanWaves];
+  if (threadIdx.x <= kPlanXcds) s_b[threadIdx.x] = threadIdx.x == 0 ? 0 : live_mb;
+  __syncthreads();
+  if (w > 0) {
+    // the block whose cost takes the running sum across x / 8 of the total is the last of XCD x - 1
+#pragma unroll
+    for (int x = 1; x < kPlanXcds; ++x) {
+      const int64_t target = (static_cast<int64_t>(total) * x + kPlanXcds - 1) / kPlanXcds;
+      if (excl < target && excl + w >= target) {
+        const int j = static_cast<int>((target - excl + 63) / 64);  // full blocks cost 64 each
+        s_b[x] = first + (j < nb ? j : nb);
+      }
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int x = 1; x <= kPlanXcds; ++x) s_b[x] = max(s_b[x], s_b[x - 1]);
+    for (int x = 1; x <= kPlanXcds; ++x) s_b[x] = min(s_b[x], s_b[x - 1] + cap_mb);
+    s_b[kPlanXcds] = live_mb;
+    for (int x = kPlanXcds - 1; x >= 1; --x) s_b[x] = max(s_b[x], s_b[x + 1] - cap_mb);
+    for (int x = 0; x <= kPlanXcds; ++x) bounds[x] = s_b[x];
+  }
+}
+
 __global__ __launch_bounds__(kScanThreads) void align_small_kernel(
     const void* __restrict__ ids, int dtype, int numel, int E, int BM, int id_bits,
     int32_t* __restrict__ sorted_ids, int64_t sorted_cap, int32_t* __restrict__ expert_ids,
-    int64_t expert_cap, int32_t* __restrict__ num_post_pad) {
+    int64_t expert_cap, int32_t* __restrict__ num_post_pad, int32_t* plan_bounds, int32_t* plan_done,
+    int plan_num_done, int plan_cap_mb) {
   extern __shared__ int lds[];
   // layout: seg_cnt[kScanWaves][E] | cum[E+1] | tot[E] | wave_tot[kScanWaves+1]
   volatile int* seg_cnt = lds;
@@ -183,6 +230,7 @@ __global__ __launch_bounds__(kScanThreads) void align_small_kernel(
   __syncthreads();
   write_blocks_and_padding(cum, tot, E, BM, numel, sorted_ids, sorted_cap, expert_ids, expert_cap,
                            num_post_pad);
+  if (plan_bounds) plan_from_counts(cum, tot, E, plan_cap_mb, plan_bounds, plan_done, plan_num_done, wave_tot);
   // per-wavefront running slots: segment prefix + expert base
   for (int e = lane; e < E; e += kWave) seg_cnt[wave * E + e] += cum[e];
   scatter_segment(ids, dtype, beg, end, E, id_bits, seg_cnt + wave * E, sorted_ids);
@@ -285,7 +333,8 @@ __global__ __launch_bounds__(kScanThreads) void align_place_kernel(
     const void* __restrict__ ids, int dtype, int64_t numel, int E, int BM, int id_bits,
     const int32_t* __restrict__ seg_cnt, int nseg, int32_t* __restrict__ sorted_ids,
     int64_t sorted_cap, int32_t* __restrict__ expert_ids, int64_t expert_cap,
-    int32_t* __restrict__ num_post_pad) {
+    int32_t* __restrict__ num_post_pad, int32_t* plan_bounds, int32_t* plan_done, int plan_num_done,
+    int plan_cap_mb) {
   extern __shared__ int lds[];
   const int nwg = gridDim.x;
   volatile int* part = lds;
@@ -364,6 +413,8 @@ __global__ __launch_bounds__(kScanThreads) void align_place_kernel(
     for (int p = beg + lane; p < end; p += kWave) sorted_ids[p] = static_cast<int32_t>(numel);
   }
   for (int64_t p = total + gtid; p < sorted_cap; p += gthreads) sorted_ids[p] = static_cast<int32_t>(numel);
+  if (plan_bounds && blockIdx.x == 0)
+    plan_from_counts(cum, tot, E, plan_cap_mb, plan_bounds, plan_done, plan_num_done, wave_tot);
   // per-wavefront running slots: ids in front of the segment + expert base
   const int sg = blockIdx.x * kScanWaves + wave;
   if (sg >= nseg) return;
@@ -402,11 +453,11 @@ MOE_EXPORT int64_t moe_align_workspace_bytes(int64_t numel, int E) {
   return moe_align_up((nseg * E + E + 1) * static_cast<int64_t>(sizeof(int32_t)), 256);
 }
 
-MOE_EXPORT int moe_align_block_size(const void* topk_ids, int ids_dtype, int64_t numel, int E,
-                                    int block_size, int32_t* sorted_token_ids, int64_t sorted_cap,
-                                    int32_t* expert_ids, int64_t expert_cap,
-                                    int32_t* num_tokens_post_pad, void* workspace,
-                                    int64_t workspace_bytes, void* stream) {
+static int align_impl(const void* topk_ids, int ids_dtype, int64_t numel, int E, int block_size,
+                      int32_t* sorted_token_ids, int64_t sorted_cap, int32_t* expert_ids,
+                      int64_t expert_cap, int32_t* num_tokens_post_pad, void* workspace,
+                      int64_t workspace_bytes, void* stream, int32_t* plan_bounds, int32_t* plan_done,
+                      int plan_num_done, int plan_cap_mb) {
   if (numel < 0 || E < 1 || block_size < 1)
     return moe_fail(MOE_ERR_ARG, "moe_align_block_size: bad sizes numel=%lld E=%d block_size=%d",
                     static_cast<long long>(numel), E, block_size);
@@ -432,7 +483,8 @@ MOE_EXPORT int moe_align_block_size(const void* topk_ids, int ids_dtype, int64_t
     const size_t lds = (static_cast<size_t>(kScanWaves) * E + (E + 1) + E + kScanWaves + 1) * sizeof(int);
     hipLaunchKernelGGL(align_small_kernel, dim3(1), dim3(kScanThreads), lds, s, topk_ids, ids_dtype,
                        static_cast<int>(numel), E, block_size, id_bits, sorted_token_ids,
-                       sorted_cap, expert_ids, expert_cap, num_tokens_post_pad);
+                       sorted_cap, expert_ids, expert_cap, num_tokens_post_pad, plan_bounds, plan_done,
+                       plan_num_done, plan_cap_mb);
     return moe_check_launch("moe_align_block_size (single workgroup)");
   }
   const int64_t need_ws = moe_align_workspace_bytes(numel, E);
@@ -450,7 +502,8 @@ MOE_EXPORT int moe_align_block_size(const void* topk_ids, int ids_dtype, int64_t
   if (place_lds <= 60 * 1024) {
     hipLaunchKernelGGL(align_place_kernel, dim3(nwg), dim3(kScanThreads), place_lds, s, topk_ids, ids_dtype,
                        numel, E, block_size, id_bits, seg_cnt, nseg, sorted_token_ids, sorted_cap,
-                       expert_ids, expert_cap, num_tokens_post_pad);
+                       expert_ids, expert_cap, num_tokens_post_pad, plan_bounds, plan_done, plan_num_done,
+                       plan_cap_mb);
     return moe_check_launch("moe_align_block_size (count + place)");
   }
   hipLaunchKernelGGL(align_scan_kernel, dim3(1), dim3(kScanThreads), 0, s, seg_cnt, nseg, E,
@@ -460,4 +513,40 @@ MOE_EXPORT int moe_align_block_size(const void* topk_ids, int ids_dtype, int64_t
                      ids_dtype, numel, E, id_bits, seg_cnt, cum,
                      sorted_token_ids);
   return moe_check_launch("moe_align_block_size");
+}
+
+MOE_EXPORT int moe_align_block_size(const void* topk_ids, int ids_dtype, int64_t numel, int E,
+                                    int block_size, int32_t* sorted_token_ids, int64_t sorted_cap,
+                                    int32_t* expert_ids, int64_t expert_cap,
+                                    int32_t* num_tokens_post_pad, void* workspace,
+                                    int64_t workspace_bytes, void* stream) {
+  return align_impl(topk_ids, ids_dtype, numel, E, block_size, sorted_token_ids, sorted_cap, expert_ids,
+                    expert_cap, num_tokens_post_pad, workspace, workspace_bytes, stream, nullptr, nullptr, 0, 0);
+}
+
+// Whether moe_align_block_size_planned can serve this size (its kernels keep per-expert
+// tables in LDS); otherwise align without a plan.
+MOE_EXPORT int moe_align_can_plan(int64_t numel, int E) {
+  if (numel < 0 || E < 1 || E > kMaxExperts) return 0;
+  if (numel <= kSmallNumel && E <= kSmallMaxExperts) return 1;
+  const int64_t nseg = numel > 0 ? (numel + kSegLen - 1) / kSegLen : 1;
+  const int64_t nwg = (nseg + kScanWaves - 1) / kScanWaves;
+  return (static_cast<size_t>(nwg + kScanWaves) * E + (E + 1) + E + kScanWaves + 1) * sizeof(int) <= 60 * 1024;
+}
+
+MOE_EXPORT int moe_align_block_size_planned(const void* topk_ids, int ids_dtype, int64_t numel, int E,
+                                            int block_size, int32_t* sorted_token_ids, int64_t sorted_cap,
+                                            int32_t* expert_ids, int64_t expert_cap,
+                                            int32_t* num_tokens_post_pad, void* workspace,
+                                            int64_t workspace_bytes, void* stream, int32_t* plan_bounds,
+                                            int32_t* plan_done, int plan_num_done, int plan_cap_mb) {
+  if (block_size != kPlanBlock || !plan_bounds || !plan_done || plan_num_done < 0 || plan_cap_mb < 1)
+    return moe_fail(MOE_ERR_ARG, "moe_align_block_size_planned: needs block_size %d and the plan buffers",
+                    kPlanBlock);
+  if (!moe_align_can_plan(numel, E))
+    return moe_fail(MOE_ERR_UNSUPPORTED, "moe_align_block_size_planned: %d experts x %lld ids is beyond the "
+                    "kernels that can plan; align without a plan", E, static_cast<long long>(numel));
+  return align_impl(topk_ids, ids_dtype, numel, E, block_size, sorted_token_ids, sorted_cap, expert_ids,
+                    expert_cap, num_tokens_post_pad, workspace, workspace_bytes, stream, plan_bounds,
+                    plan_done, plan_num_done, plan_cap_mb);
 }

@@ -1652,6 +1652,24 @@ MOE_EXPORT int64_t moe_fused_experts_workspace_bytes(int T, int H, int I, int E,
   return bytes + moe_align_up((sorted_cap + kBigBM - 1) / kBigBM * 4, 256) + 256;
 }
 
+// Where in the workspace of a moe_fused_experts call of these sizes the per-XCD ranges (9
+// int32) and the per-block counters sit, for moe_align_block_size_planned.  Returns 1 when
+// such a call uses them (blocks that are multiples of 256 slots, 16-bit activations), else 0.
+MOE_EXPORT int moe_fused_experts_plan_layout(int T, int H, int I, int E, int K, int block_size,
+                                             int act_dtype, int weight_dtype, int64_t* bounds_offset,
+                                             int64_t* done_offset, int32_t* num_done, int32_t* cap_mb) {
+  if (T < 1 || block_size % kBigBM != 0 || act_dtype == MOE_F32) return 0;
+  const int64_t need_ws = moe_fused_experts_workspace_bytes(T, H, I, E, K, block_size, act_dtype, weight_dtype);
+  if (need_ws <= 0) return 0;
+  const int64_t sorted_cap = static_cast<int64_t>(T) * K + static_cast<int64_t>(E) * (block_size - 1);
+  const int64_t nd = (sorted_cap + kBigBM - 1) / kBigBM;
+  *bounds_offset = need_ws - 256;
+  *done_offset = need_ws - 256 - moe_align_up(nd * 4, 256);
+  *num_done = static_cast<int32_t>(nd);
+  *cap_mb = big_plan_cap(sorted_cap);
+  return 1;
+}
+
 MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   if (!a) return moe_fail(MOE_ERR_ARG, "fused_experts: null argument block");
   if (a->T < 0 || a->H < 1 || a->I < 1 || a->E < 1 || a->K < 1)
@@ -1722,10 +1740,12 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
     int32_t* bounds = reinterpret_cast<int32_t*>(static_cast<char*>(a->workspace) + need_ws - 256);
     const int num_done = static_cast<int>((a->sorted_cap + kBigBM - 1) / kBigBM);
     plan_done = bounds - moe_align_up(static_cast<int64_t>(num_done) * 4, 256) / 4;
-    hipLaunchKernelGGL(big_plan_kernel, dim3(1), dim3(kPlanThreads), 0, s, a->sorted_token_ids,
-                       a->num_tokens_post_pad, static_cast<int>(numel), big_plan_cap(a->sorted_cap), bounds,
-                       plan_done, num_done);
-    if (int rc0 = moe_check_launch("fused_experts (XCD ranges)")) return rc0;
+    if (!(a->passes & 16)) {  // bit 16: moe_align_block_size_planned already left the plan here
+      hipLaunchKernelGGL(big_plan_kernel, dim3(1), dim3(kPlanThreads), 0, s, a->sorted_token_ids,
+                         a->num_tokens_post_pad, static_cast<int>(numel), big_plan_cap(a->sorted_cap), bounds,
+                         plan_done, num_done);
+      if (int rc0 = moe_check_launch("fused_experts (XCD ranges)")) return rc0;
+    }
     plan_bounds = bounds;
   }
   p.xcd_bounds = plan_bounds;
@@ -1734,7 +1754,7 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.bias = a->w13_bias; p.bias_stride_e = 2LL * a->I;
   p.c = inter; p.ldc = a->I; p.Kd = a->H; p.N = a->I; p.a_by_slot = 0;
   p.mul_weight = a->apply_router_weight_on_input ? 1 : 0;
-  const int passes = a->passes ? a->passes : 7;
+  const int passes = (a->passes & 7) ? a->passes : (a->passes | 7);
   int rc = MOE_OK;
   if (plan_bounds && !fp8 && (passes & 3) == 3 && !(passes & 8)) {
     // 16-bit dtypes on the large-tile kernel: both passes in one launch

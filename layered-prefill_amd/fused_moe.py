@@ -22,14 +22,39 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
     [numel + E*(block_size-1)], expert_ids [ceil(that / block_size)],
     num_tokens_post_padded [1]), all int32 on topk_ids' device.  The kernel
     writes every element of all three, so nothing is pre-filled here."""
+    return _align_block_size(topk_ids, block_size, num_experts, None)
+
+
+def _align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: int, plan
+                      ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``moe_align_block_size``; with ``plan`` (see ``ops.align_block_size_planned``)
+    the alignment also prepares the launch of the expert GEMMs that follows."""
     max_num_tokens_padded = topk_ids.numel() + num_experts * (block_size - 1)
     sorted_ids = torch.empty((max_num_tokens_padded,), dtype=torch.int32, device=topk_ids.device)
     max_num_m_blocks = cdiv(max_num_tokens_padded, block_size)
     expert_ids = torch.empty((max_num_m_blocks,), dtype=torch.int32, device=topk_ids.device)
     num_tokens_post_pad = torch.empty((1), dtype=torch.int32, device=topk_ids.device)
-    ops.moe_align_block_size(topk_ids, num_experts, block_size, sorted_ids, expert_ids,
-                             num_tokens_post_pad)
+    ops.align_block_size_planned(topk_ids, num_experts, block_size, sorted_ids, expert_ids,
+                                 num_tokens_post_pad, plan)
     return sorted_ids, expert_ids, num_tokens_post_pad
+
+
+def _plan_in_workspace(workspace: torch.Tensor, T: int, H: int, I: int, E: int, K: int, block_size: int,
+                       act_code: int, weight_code: int, numel: int):
+    """Where the alignment may leave the large-tile kernel's per-XCD ranges and
+    cleared counters inside ``workspace`` (the tuple ``ops.align_block_size_planned``
+    takes), or None when this call has no use for them."""
+    import ctypes
+    L = lib()
+    if block_size != 256 or not L.moe_align_can_plan(numel, E):
+        return None
+    b_off, d_off = ctypes.c_int64(), ctypes.c_int64()
+    n_done, cap_mb = ctypes.c_int32(), ctypes.c_int32()
+    if not L.moe_fused_experts_plan_layout(T, H, I, E, K, block_size, act_code, weight_code, ctypes.byref(b_off),
+                                           ctypes.byref(d_off), ctypes.byref(n_done), ctypes.byref(cap_mb)):
+        return None
+    base = workspace.data_ptr()
+    return (base + b_off.value, base + d_off.value, n_done.value, cap_mb.value)
 
 
 def try_get_optimal_moe_config(w1_shape, w2_shape, top_k: int, dtype: Optional[str], M: int,
@@ -281,10 +306,20 @@ def fused_experts_impl(hidden_states: torch.Tensor,
         bm = config["BLOCK_SIZE_M"]
         curr_ids = topk_ids[begin:end]
         curr_w = topk_weights[begin:end]
-        sorted_token_ids, expert_ids, num_tokens_post_padded = moe_align_block_size(
-            curr_ids, bm, global_num_experts)
+        # the workspace first: with blocks of 256 the alignment also leaves the large-tile
+        # kernel's per-XCD ranges and cleared counters in it (one launch less)
+        ws_bytes = L.moe_fused_experts_workspace_bytes(tokens_in_chunk, w1.size(2), N // 2, global_num_experts,
+                                                       top_k_num, bm, act_code, weight_code)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        plan = None
+        if global_num_experts == E:
+            plan = _plan_in_workspace(workspace, tokens_in_chunk, w1.size(2), N // 2, E, top_k_num, bm,
+                                      act_code, weight_code, curr_ids.numel())
+        sorted_token_ids, expert_ids, num_tokens_post_padded = _align_block_size(
+            curr_ids, bm, global_num_experts, plan)
         launch_fused_experts(hidden_states[begin:end], out_hidden_states[begin:end], w1, w2,
                              w1_bias, w2_bias, w1_scale, w2_scale, curr_w, sorted_token_ids,
                              expert_ids, num_tokens_post_padded, bm, activation,
-                             apply_router_weight_on_input, weight_code=weight_code)
+                             apply_router_weight_on_input, weight_code=weight_code,
+                             workspace=workspace, passes=16 if plan is not None else 0)
     return out_hidden_states

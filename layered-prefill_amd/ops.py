@@ -106,6 +106,17 @@ def moe_align_block_size(topk_ids: torch.Tensor, num_experts: int, block_size: i
                          sorted_token_ids: torch.Tensor, experts_ids: torch.Tensor,
                          num_tokens_post_pad: torch.Tensor) -> None:
     """csrc/moe_align_block_size_kernels.cu:239-291."""
+    align_block_size_planned(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids,
+                             num_tokens_post_pad, None)
+
+
+def align_block_size_planned(topk_ids: torch.Tensor, num_experts: int, block_size: int,
+                             sorted_token_ids: torch.Tensor, experts_ids: torch.Tensor,
+                             num_tokens_post_pad: torch.Tensor, plan) -> None:
+    """``moe_align_block_size`` with an optional ``plan`` (not in the reference):
+    ``(bounds_ptr, done_ptr, num_done, cap_mb)`` inside the workspace of the
+    ``moe_fused_experts`` call that follows, for the entry point that also leaves
+    the large-tile kernel's per-XCD ranges and cleared counters there."""
     require_gpu_tensor(topk_ids, "topk_ids")
     if topk_ids.dtype not in _lib.ID_DTYPE_CODE:
         raise RuntimeError(f"moe_align_block_size_kernel not implemented for '{topk_ids.dtype}'")
@@ -121,14 +132,16 @@ def moe_align_block_size(topk_ids: torch.Tensor, num_experts: int, block_size: i
     L = lib()
     ws_bytes = L.moe_align_workspace_bytes(numel, num_experts)
     ws = _align_workspace(ws_bytes, topk_ids.device) if ws_bytes else None
+    common = (topk_ids.data_ptr(), _lib.ID_DTYPE_CODE[topk_ids.dtype], numel, num_experts, block_size,
+              sorted_token_ids.data_ptr(), sorted_token_ids.numel(), experts_ids.data_ptr(),
+              experts_ids.numel(), num_tokens_post_pad.data_ptr(),
+              ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
+              stream_ptr(topk_ids.device))
     with torch.cuda.device(topk_ids.device):
-        check(L.moe_align_block_size(topk_ids.data_ptr(), _lib.ID_DTYPE_CODE[topk_ids.dtype], numel,
-                                     num_experts, block_size, sorted_token_ids.data_ptr(),
-                                     sorted_token_ids.numel(), experts_ids.data_ptr(),
-                                     experts_ids.numel(), num_tokens_post_pad.data_ptr(),
-                                     ws.data_ptr() if ws is not None else None,
-                                     ws.numel() if ws is not None else 0,
-                                     stream_ptr(topk_ids.device)))
+        if plan is None:
+            check(L.moe_align_block_size(*common))
+        else:
+            check(L.moe_align_block_size_planned(*common, *plan))
 
 
 def _act_args(out: torch.Tensor, input: torch.Tensor):

@@ -276,3 +276,48 @@ def test_rms_norm_module_mirrors_the_reference_interface(moe, oracle, dev):
     with pytest.raises(RuntimeError, match="hidden_size"):
         moe.ops.rms_norm(torch.empty(2, 4, 8, device=dev), torch.empty(2, 4, 8, device=dev),
                          torch.ones(8, device=dev), 1e-6)
+
+
+@pytest.mark.parametrize("T,E,K,skew", [(256, 128, 8, True), (8448, 128, 8, True), (3000, 64, 1, False),
+                                        (40, 8, 2, False), (5000, 384, 4, True), (70, 128, 8, True)])
+def test_planned_alignment_leaves_the_plan_of_the_plan_kernel(moe, oracle, dev, T, E, K, skew):
+    """With blocks of 256 the alignment can also leave, in the workspace of the expert call
+    that follows, the per-XCD block ranges and cleared counters which that call otherwise
+    computes with a launch of its own (from the aligned ids).  Both must be the same plan,
+    and the alignment outputs must not change."""
+    fm, L = moe.fused_moe, moe._lib.lib()
+    H, I, bm = 256, 128, 256
+    code = moe._lib.DTYPE_CODE[torch.bfloat16]
+    if skew:
+        ids = _skewed_ids(T * K, E, 5 * T + E).view(T, K)
+    else:
+        ids = torch.randint(0, E, (T, K), generator=torch.Generator().manual_seed(T + E)).to(torch.int32)
+    ids = ids.to(dev)
+    ws = torch.full((L.moe_fused_experts_workspace_bytes(T, H, I, E, K, bm, code, code),), 0x5a,
+                    dtype=torch.uint8, device=dev)
+    plan = fm._plan_in_workspace(ws, T, H, I, E, K, bm, code, code, ids.numel())
+    assert plan is not None
+    b_ptr, d_ptr, n_done, cap_mb = plan
+    base = ws.data_ptr()
+    got = fm._align_block_size(ids, bm, E, plan)
+    want = oracle.moe_align_block_size(ids.cpu(), bm, E)
+    assert all(torch.equal(a.cpu(), b) for a, b in zip(got, want))
+    words = ws.view(torch.int32)
+    bounds = words[(b_ptr - base) // 4:(b_ptr - base) // 4 + 9].cpu()
+    done = words[(d_ptr - base) // 4:(d_ptr - base) // 4 + n_done].cpu()
+    assert int(done.abs().max()) == 0
+    # the plan kernel on the same aligned ids, in a second workspace (gate-up pass only)
+    ws2 = torch.full_like(ws, 0x5a)
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(T, H, generator=g).bfloat16().to(dev)
+    w13 = (torch.randn(E, 2 * I, H, generator=g) * 0.05).bfloat16().to(dev)
+    w2 = (torch.randn(E, H, I, generator=g) * 0.05).bfloat16().to(dev)
+    tw = torch.rand(T, K, generator=g).to(dev)
+    fm.launch_fused_experts(x, torch.empty_like(x), w13, w2, None, None, None, None, tw, *got, bm,
+                            workspace=ws2, passes=1)
+    torch.cuda.synchronize()
+    bounds2 = ws2.view(torch.int32)[(b_ptr - base) // 4:(b_ptr - base) // 4 + 9].cpu()
+    assert torch.equal(bounds, bounds2), (bounds.tolist(), bounds2.tolist())
+    live = int(got[2].item()) // 256
+    assert bounds[0] == 0 and bounds[8] == live and bool((bounds[1:] >= bounds[:-1]).all())
+    assert int((bounds[1:] - bounds[:-1]).max()) <= cap_mb
