@@ -1086,7 +1086,8 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
     const int lo = p.xcd_bounds[blockIdx.x % kXcds], hi = p.xcd_bounds[blockIdx.x % kXcds + 1];
     mb = lo + xslot / p.num_n_tiles;
     nt = xslot % p.num_n_tiles;
-    if (mb >= hi) return;
+    // the second test keeps a plan that was never written from sending a tile out of range
+    if (mb >= hi || lo < 0 || mb >= p.num_m_blocks) return;
   } else {
   const int npp = *p.num_post_pad;
   const int live_mb = (npp + kBigBM - 1) / kBigBM;
@@ -1126,7 +1127,7 @@ __global__ __launch_bounds__(kThreads, 1) void big_fused_kernel(const GemmParams
   const int n1 = cap_mb * p1.num_n_tiles;
   if (xslot < n1) {
     const int mb = lo + xslot / p1.num_n_tiles, nt = xslot % p1.num_n_tiles;
-    if (mb >= hi) return;
+    if (mb >= hi || lo < 0 || mb >= p1.num_m_blocks) return;  // (an unwritten plan must not send a tile out of range)
     big_tile<Mma, true>(p1, mb, nt, smem);
     // every store of this tile has been taken by the L2 before the count goes up
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -1135,7 +1136,7 @@ __global__ __launch_bounds__(kThreads, 1) void big_fused_kernel(const GemmParams
   } else {
     const int j = xslot - n1;
     const int mb = lo + j / p2.num_n_tiles, nt = j % p2.num_n_tiles;
-    if (mb >= hi) return;
+    if (mb >= hi || lo < 0 || mb >= p1.num_m_blocks) return;
     if (threadIdx.x == 0) {
       int spins = 0;
       while (__hip_atomic_load(done + mb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < p1.num_n_tiles &&
