@@ -4,6 +4,7 @@ defaults, assertions and return values) on top of libmoe_gfx950.so.
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Optional, Tuple
 
 import torch
@@ -44,7 +45,6 @@ def _plan_in_workspace(workspace: torch.Tensor, T: int, H: int, I: int, E: int, 
     """Where the alignment may leave the large-tile kernel's per-XCD ranges and
     cleared counters inside ``workspace`` (the tuple ``ops.align_block_size_planned``
     takes), or None when this call has no use for them."""
-    import ctypes
     L = lib()
     if block_size != 256 or not L.moe_align_can_plan(numel, E):
         return None
