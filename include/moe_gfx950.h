@@ -13,6 +13,9 @@
  *  - `stream` is a hipStream_t passed as void* (NULL = the null stream).
  *  - Return value 0 = enqueued; negative = rejected, nothing enqueued.
  *    `moe_last_error()` then returns a thread-local, human-readable reason.
+ *  - Host-side state: the per-device "large LDS opted in" flags of the kernels and the
+ *    wait limit of moe_fused_experts_set_wait_limit, all atomics; entry points may be
+ *    called from several host threads.
  *  - Scratch memory comes from the caller (`workspace`), sized by the
  *    matching `*_workspace_bytes` function, 256-byte aligned.
  */
@@ -37,7 +40,9 @@ enum MoeError {
   MOE_ERR_ARG = -1,        /* bad shape / null pointer / unsupported value */
   MOE_ERR_UNSUPPORTED = -2,/* valid request this build has no kernel for    */
   MOE_ERR_WORKSPACE = -3,  /* workspace missing or too small                */
-  MOE_ERR_LAUNCH = -4      /* hipLaunchKernel reported an error             */
+  MOE_ERR_LAUNCH = -4,     /* hipLaunchKernel reported an error             */
+  MOE_ERR_HANDOFF = -5     /* moe_fused_experts_status: a bounded device-side wait of the
+                              previous call expired; its output holds NaN rows */
 };
 
 const char* moe_last_error(void);
@@ -151,7 +156,10 @@ typedef struct MoeFusedExpertsArgs {
   /* sizes */
   int32_t T, H, I, E, K;
   int32_t block_size;        /* the block_size the alignment was made with          */
-  int64_t sorted_cap;        /* numel + E*(block_size-1)                             */
+  int64_t sorted_cap;        /* length of sorted_token_ids, >= T*K + E*(block_size-1); the
+                                alignment must have been made with the same E and
+                                block_size, so nothing lives beyond that length and a
+                                longer buffer's surplus is ignored                   */
   int32_t act_dtype;         /* MoeDtype of x / out / biases                         */
   int32_t weight_dtype;      /* MoeDtype of w13 / w2 (MOE_E4M3 selects the fp8 path) */
   int32_t activation;        /* MoeActivation                                        */
@@ -170,6 +178,24 @@ typedef struct MoeFusedExpertsArgs {
 int64_t moe_fused_experts_workspace_bytes(int T, int H, int I, int E, int K, int block_size,
                                           int act_dtype, int weight_dtype);
 int moe_fused_experts(const MoeFusedExpertsArgs* args);
+
+/* No counterpart in the reference (its two Triton launches need no hand-off).  With 16-bit
+ * dtypes and blocks of 256 slots moe_fused_experts enqueues both GEMM passes as one launch,
+ * in which the down tiles of a 256-slot block wait on the device, for a bounded number of
+ * polls, until the gate-up tiles of that block have been counted in.  A down tile whose
+ * wait expires does not compute: it fills its rows of the result with NaN (which reach
+ * `out` through the top-k combine) and counts itself in a status word of the workspace that
+ * the next call's plan clears.  moe_fused_experts_status, given the argument block of the
+ * most recent moe_fused_experts call on that workspace, copies the word to the host,
+ * WAITS FOR `stream` (the only entry point of this library that synchronises) and returns 0,
+ * or MOE_ERR_HANDOFF when waits expired (moe_last_error says how many).  Calls that do not
+ * use the one-launch form return 0 without touching the device. */
+int moe_fused_experts_status(const MoeFusedExpertsArgs* args);
+/* Polls (about a microsecond each) a down tile waits before it gives up; default 2,000,000.
+ * Process-wide, read at every moe_fused_experts call; returns the previous value.  0 makes
+ * every down tile that finds its block incomplete give up at once: the host-forced error
+ * path for tests (all kernels still exit normally). */
+int moe_fused_experts_set_wait_limit(int polls);
 /* Offsets into the workspace (and sizes) of the plan that moe_align_block_size_planned
  * writes for a moe_fused_experts call of these sizes; returns 1 when the call uses one. */
 int moe_fused_experts_plan_layout(int T, int H, int I, int E, int K, int block_size, int act_dtype,

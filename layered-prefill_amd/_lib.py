@@ -28,6 +28,7 @@ EXPORTS = (
     "moe_fused_experts_workspace_bytes", "moe_fused_experts", "moe_preferred_block_size",
     "moe_quant_rows_e4m3", "moe_gate_topk_softmax", "moe_add_rms_norm",
     "moe_align_can_plan", "moe_align_block_size_planned", "moe_fused_experts_plan_layout",
+    "moe_fused_experts_status", "moe_fused_experts_set_wait_limit",
 )
 
 
@@ -92,6 +93,10 @@ def _declare(L: ctypes.CDLL) -> None:
     L.moe_fused_experts_workspace_bytes.argtypes = [i32] * 8
     L.moe_fused_experts.restype = i32
     L.moe_fused_experts.argtypes = [ctypes.POINTER(MoeFusedExpertsArgs)]
+    L.moe_fused_experts_status.restype = i32
+    L.moe_fused_experts_status.argtypes = [ctypes.POINTER(MoeFusedExpertsArgs)]
+    L.moe_fused_experts_set_wait_limit.restype = i32
+    L.moe_fused_experts_set_wait_limit.argtypes = [i32]
     L.moe_preferred_block_size.restype = i32
     L.moe_preferred_block_size.argtypes = [i32] * 5
     L.moe_quant_rows_e4m3.restype = i32

@@ -147,13 +147,15 @@ __device__ __forceinline__ void scatter_segment(const void* ids, int dtype, int6
 // per-expert counts instead, for an alignment with blocks of 256 slots: the m-block
 // ranges [bounds[x], bounds[x+1]) of the 8 XCDs with equal estimated work (a block costs
 // 36 / 45 / 62 / 64 with at most 32 / at most 64 / fewer than 256 / 256 real slots), no range
-// longer than cap_mb, and the per-block counters of the one-launch form cleared.  Saves the
+// longer than cap_mb, and the per-block counters and the status word of the one-launch form
+// cleared.  Saves the
 // large-tile path a launch.  Called by all kScanThreads threads; contains barriers.
 constexpr int kPlanBlock = 256, kPlanXcds = 8;
 __device__ void plan_from_counts(const volatile int* cum, const volatile int* tot, int E, int cap_mb,
                                  int32_t* bounds, int32_t* done, int num_done, volatile int* wave_tot) {
   __shared__ int s_b[kPlanXcds + 1];
   for (int i = threadIdx.x; i < num_done; i += kScanThreads) done[i] = 0;
+  if (threadIdx.x == 0) bounds[kMoeStatusWord] = 0;  // expired waits of the one-launch form
   const int live_mb = cum[E] / kPlanBlock;
   int w = 0, nb = 0, first = 0;
   if (static_cast<int>(threadIdx.x) < E) {

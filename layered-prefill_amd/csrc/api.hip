@@ -22,6 +22,18 @@ int moe_check_launch(const char* what) {
   return moe_fail(MOE_ERR_LAUNCH, "%s: kernel launch failed: %s", what, hipGetErrorString(e));
 }
 
+int moe_opt_in_lds(MoeLdsOptIn& flags, const void* kernel, int lds_bytes, const char* what) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) dev = 0;
+  const bool tracked = dev < kMoeMaxDevices;  // devices beyond the table set the attribute on every call
+  if (tracked && flags.done[dev].load(std::memory_order_acquire)) return MOE_OK;
+  hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+  if (e != hipSuccess)
+    return moe_fail(MOE_ERR_LAUNCH, "%s: cannot reserve %d B of LDS: %s", what, lds_bytes, hipGetErrorString(e));
+  if (tracked) flags.done[dev].store(true, std::memory_order_release);  // two threads setting it twice is harmless
+  return MOE_OK;
+}
+
 MOE_EXPORT const char* moe_last_error(void) { return g_last_error; }
 
 MOE_EXPORT int moe_abi_version(void) { return 1; }

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/moe_gfx950.h"
 
 #define MOE_EXPORT extern "C" __attribute__((visibility("default")))
@@ -17,6 +19,19 @@ int moe_check_launch(const char* what);
 int moe_quant_slot_rows_e4m3(const void* w, int src_dtype, int64_t rows, int cols, uint8_t* q,
                              float* scales, const int32_t* row_ids, int64_t id_count, int numel,
                              void* stream);
+
+// Dynamic LDS above 64 KB must be opted into once per kernel and device.  One MoeLdsOptIn
+// per kernel instantiation (a zero-initialised static); moe_opt_in_lds sets the attribute on
+// the current device when it has not been set there yet.  Safe from several host threads.
+constexpr int kMoeMaxDevices = 64;
+struct MoeLdsOptIn {
+  std::atomic<bool> done[kMoeMaxDevices];
+};
+int moe_opt_in_lds(MoeLdsOptIn& flags, const void* kernel, int lds_bytes, const char* what);
+
+// int32 index, inside the 256-byte table of per-XCD ranges at the end of a moe_fused_experts
+// workspace, of the count of expired waits of the one-launch form (cleared with the plan).
+constexpr int kMoeStatusWord = 16;
 
 static inline int64_t moe_align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
@@ -67,13 +82,18 @@ struct ElemF16 {
 // exp in fp32 as a fixed sequence of IEEE operations: Cody-Waite reduction by
 // ln2 (two constants), degree-6 polynomial evaluated with fused multiply-adds,
 // scaling through the exponent field.  <= 2 ulp.  Inputs above 88 give +inf,
-// inputs below -87 give 0 (no subnormal results).  Translation units that use
-// it are compiled with -ffp-contract=off so that no other operation is fused.
+// inputs below -104 give 0; between about -87.3 and -104 the result is
+// subnormal, as CUDA's expf returns it when built without flush-to-zero (the
+// reference's build, setup.py:46-47): such results are scaled in two steps, by
+// 2^(n+64) through the exponent field (exact) and by one multiplication with
+// 2^-64, which rounds once.  gfx950 code objects keep fp32 subnormals (denormal
+// mode 3).  Translation units that use it are compiled with -ffp-contract=off
+// so that no other operation is fused.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float moe_expf(float x) {
   if (x != x) return x;
   if (x > 88.0f) return __builtin_inff();
-  if (x < -87.0f) return 0.0f;
+  if (x < -104.0f) return 0.0f;
   float n = __builtin_rintf(x * 1.44269504088896341f);
   float r = __builtin_fmaf(n, -0.693359375f, x);
   r = __builtin_fmaf(n, 2.12194440e-4f, r);
@@ -87,6 +107,10 @@ __device__ __forceinline__ float moe_expf(float x) {
   p = __builtin_fmaf(p, r2, r);
   p = p + 1.0f;
   int32_t ni = static_cast<int32_t>(n);
+  if (ni < -125) {
+    const float t = __uint_as_float(__float_as_uint(p) + (static_cast<uint32_t>(ni + 64) << 23));
+    return t * 5.42101086242752217e-20f;  // 2^-64
+  }
   return __uint_as_float(__float_as_uint(p) + (static_cast<uint32_t>(ni) << 23));
 }
 

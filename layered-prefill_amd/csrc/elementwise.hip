@@ -101,7 +101,12 @@ __device__ __forceinline__ uint32_t f32x2_to_e4m3(float a, float b) {
   return static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false)) & 0xffffu;
 }
 
-// One wavefront per row: s = amax|row| / 448 (1 for an all-zero row),
+// Smallest row scale: a row whose largest magnitude is tiny but not zero would get
+// a scale whose reciprocal overflows (amax below about 1.3e-36); from 2^-100 down
+// the scale stays 2^-100 and the row's codes are simply small.
+constexpr float kMinScale = 7.888609052210118e-31f;  // 2^-100
+
+// One wavefront per row: s = max(amax|row| / 448, 2^-100) (1 for an all-zero row),
 // q = e4m3(row * (1 / s)): one correctly rounded division per row, then one
 // multiplication per element (a division per element made the kernel
 // VALU-bound: 48 us for 67584 x 768 against 28 us of memory time).
@@ -118,7 +123,7 @@ __global__ __launch_bounds__(kThreads) void quant_rows_e4m3_kernel(
   for (int c = lane; c < cols; c += kWave) amax = fmaxf(amax, fabsf(El::ld(src[c])));
 #pragma unroll
   for (int m = 32; m > 0; m /= 2) amax = fmaxf(amax, __shfl_xor(amax, m, kWave));
-  const float s = amax > 0.f ? amax / 448.f : 1.f;
+  const float s = amax > 0.f ? fmaxf(amax / 448.f, kMinScale) : 1.f;
   if (lane == 0) scales[row] = s;
   const float inv = 1.0f / s;
   for (int c = lane; c < cols; c += kWave) q[row * cols + c] = f32_to_e4m3(El::ld(src[c]) * inv);
@@ -152,7 +157,7 @@ __global__ __launch_bounds__(kThreads) void quant_rows_e4m3_vec_kernel(
   }
 #pragma unroll
   for (int m = 32; m > 0; m /= 2) amax = fmaxf(amax, __shfl_xor(amax, m, kWave));
-  const float s = amax > 0.f ? amax / 448.f : 1.f;
+  const float s = amax > 0.f ? fmaxf(amax / 448.f, kMinScale) : 1.f;
   if (lane == 0) scales[row] = s;
   const float inv = 1.0f / s;
   uint2* dst = reinterpret_cast<uint2*>(q + row * cols);

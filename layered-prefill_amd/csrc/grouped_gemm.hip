@@ -413,7 +413,8 @@ constexpr int kEpiWaveBytes = 128 * kEpiRowBytes;
 constexpr int kBigLdsBytes = 4 * kEpiWaveBytes;    // epilogue staging, reuses the ring
 constexpr int kBigSideBytes = 5 * kBigBM * 4;      // per slot: token id, routed weight, fp8 row scale; per weight row: fp8 scale, bias
 constexpr int kBigLdsTotal = kBigUnits * kBigUnitBytes;  // the whole 160 KB of the CU
-static_assert(kBigLdsBytes + kBigSideBytes + 16 <= kBigLdsTotal, "epilogue staging must fit in the ring");
+static_assert(kBigLdsBytes + kBigSideBytes + 32 <= kBigLdsTotal, "epilogue staging must fit in the ring");
+constexpr int kBigStatusWord = kMoeStatusWord;
 
 typedef __attribute__((address_space(3))) char lds_char;
 
@@ -1111,16 +1112,34 @@ __global__ __launch_bounds__(kThreads, 1) void big_gemm_kernel(const GemmParams 
 // the gate-up tiles of its m-block range, then the down tiles of the same range,
 // so its CUs move on to down tiles while the last gate-up tiles are still running
 // instead of idling through the tail of one launch and the ramp of the next.
-// A down tile reads intermediate rows that gate-up tiles of the same XCD wrote:
-// they meet in that XCD's L2.  done[mb] counts the finished gate-up tiles of
-// m-block mb (zeroed by big_plan_kernel); a down tile starts once all of them are
-// in, which at its place in the order is normally long the case.  The wait is
-// bounded (spin_limit polls of about a microsecond), so the grid drains even if
-// the order were not what is assumed.
+// done[mb] counts the finished gate-up tiles of m-block mb (zeroed by the plan
+// step); a down tile starts once all of them are in, which at its place in the
+// order is normally long the case.  The hand-off is a release/acquire pair at
+// device scope: the gate-up workgroup's stores are complete and written back
+// before its count goes up, and the down tile's loads come after it has seen
+// the full count, so the result does not depend on which XCD either side ran on.
+// The wait is bounded (spin_limit polls of about a microsecond) so that the grid
+// drains whatever happens.  A down tile whose wait expires does not multiply a
+// partly written intermediate: it fills its output rows with NaN, which the top-k
+// combine carries into `out`, and adds one to the status word that
+// moe_fused_experts_status reads back.
+template <typename El>
+__device__ __forceinline__ void big_poison_tile(const GemmParams& p, int mb, int nt) {
+  using S = typename El::S;
+  const int64_t slot = static_cast<int64_t>(mb) * kBigBM + threadIdx.x;
+  if (slot >= p.sorted_cap) return;
+  const int tok = p.sorted_ids[slot];
+  if (tok >= p.numel) return;
+  const S nan = sizeof(S) == 2 ? El::st(__builtin_nanf("")) : S{};
+  S* row = static_cast<S*>(p.c) + static_cast<int64_t>(tok) * p.ldc;
+  const int n0 = nt * kBigBNW;
+  for (int n = n0; n < n0 + kBigBNW && n < p.N; ++n) row[n] = nan;
+}
+
 template <typename Mma>
 __global__ __launch_bounds__(kThreads, 1) void big_fused_kernel(const GemmParams p1, const GemmParams p2,
                                                                 int32_t* __restrict__ done, int cap_mb,
-                                                                int spin_limit) {
+                                                                int spin_limit, int32_t* __restrict__ status) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const int x = blockIdx.x % kXcds, xslot = blockIdx.x / kXcds;
   const int lo = p1.xcd_bounds[x], hi = p1.xcd_bounds[x + 1];
@@ -1129,21 +1148,31 @@ __global__ __launch_bounds__(kThreads, 1) void big_fused_kernel(const GemmParams
     const int mb = lo + xslot / p1.num_n_tiles, nt = xslot % p1.num_n_tiles;
     if (mb >= hi || lo < 0 || mb >= p1.num_m_blocks) return;  // (an unwritten plan must not send a tile out of range)
     big_tile<Mma, true>(p1, mb, nt, smem);
-    // every store of this tile has been taken by the L2 before the count goes up
+    // every store of this workgroup has been taken by the L2 before the barrier; the release
+    // then makes them visible device-wide before the count goes up
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (threadIdx.x == 0) __hip_atomic_fetch_add(done + mb, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (threadIdx.x == 0) __hip_atomic_fetch_add(done + mb, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
   } else {
     const int j = xslot - n1;
     const int mb = lo + j / p2.num_n_tiles, nt = j % p2.num_n_tiles;
     if (mb >= hi || lo < 0 || mb >= p1.num_m_blocks) return;
+    int* s_flag = reinterpret_cast<int*>(smem + kBigLdsBytes + kBigSideBytes + 16);
     if (threadIdx.x == 0) {
       int spins = 0;
-      while (__hip_atomic_load(done + mb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < p1.num_n_tiles &&
+      bool ready;
+      while (!(ready = __hip_atomic_load(done + mb, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) >= p1.num_n_tiles) &&
              spins++ < spin_limit)
         __builtin_amdgcn_s_sleep(32);
+      *s_flag = ready ? 1 : 0;
     }
     __syncthreads();
+    if (*s_flag == 0) {  // workgroup-uniform
+      big_poison_tile<typename Mma::El>(p2, mb, nt);
+      if (threadIdx.x == 0) __hip_atomic_fetch_add(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return;
+    }
+    // (the flag word lies in ring slot 4, which big_tile writes only behind its own barriers)
     big_tile<Mma, false>(p2, mb, nt, smem);
   }
 }
@@ -1164,8 +1193,9 @@ __global__ __launch_bounds__(kPlanThreads) void big_plan_kernel(const int32_t* _
                                                                 int numel, int cap_mb, int32_t* __restrict__ bounds,
                                                                 int32_t* __restrict__ done, int num_done) {
   __shared__ int s_wave[kPlanThreads / kWave + 1];
-  // per-m-block counters of the one-launch form start at zero
+  // per-m-block counters of the one-launch form start at zero, and so does the count of expired waits
   for (int i = threadIdx.x; i < num_done; i += kPlanThreads) done[i] = 0;
+  if (threadIdx.x == 0) bounds[kBigStatusWord] = 0;
   __shared__ int s_b[kXcds + 1];
   const int live_mb = (*num_post_pad + kBigBM - 1) / kBigBM;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -1470,6 +1500,10 @@ int launch_stream(GemmParams& p, int64_t sorted_cap, hipStream_t s) {
   return moe_check_launch(GATED ? "fused_experts (gate-up pass)" : "fused_experts (down pass)");
 }
 
+// Polls a down tile of the one-launch form waits for its m-block's gate-up tiles (about a
+// microsecond each): two seconds by default, far beyond any launch of this kernel.
+static std::atomic<int> g_wait_limit{2000000};
+
 // Longest m-block range big_plan_kernel may give an XCD: twice the average (a range of
 // weight-streaming blocks only, at about half the cost each), never more than all blocks.
 static int big_plan_cap(int64_t sorted_cap) {
@@ -1482,14 +1516,8 @@ template <typename Mma, bool GATED>
 int launch_big(GemmParams& p, int64_t sorted_cap, hipStream_t s) {
   constexpr int lds = kBigLdsTotal;
   auto kern = big_gemm_kernel<Mma, GATED>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess)
-      return moe_fail(MOE_ERR_LAUNCH, "fused_experts: cannot reserve %d B of LDS: %s", lds, hipGetErrorString(e));
-    attr_set = true;
-  }
+  static MoeLdsOptIn opted;  // per instantiation
+  if (int rc = moe_opt_in_lds(opted, reinterpret_cast<const void*>(kern), lds, "fused_experts")) return rc;
   p.num_m_blocks = static_cast<int>((sorted_cap + kBigBM - 1) / kBigBM);
   p.num_n_tiles = (p.N + (GATED ? 128 : 256) - 1) / (GATED ? 128 : 256);
   const int64_t tiles = static_cast<int64_t>(p.num_m_blocks) * p.num_n_tiles;
@@ -1505,14 +1533,8 @@ template <typename Mma, int BM, int BNW, int WAVES_M, bool GATED>
 int launch(const GemmParams& p, hipStream_t s) {
   constexpr int lds = 2 * (BM + BNW) * kRowBytes;
   auto kern = grouped_gemm_kernel<Mma, BM, BNW, WAVES_M, GATED>;
-  static bool attr_set = false;  // per instantiation; dynamic LDS above 64 KB must be opted into
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess)
-      return moe_fail(MOE_ERR_LAUNCH, "fused_experts: cannot reserve %d B of LDS: %s", lds, hipGetErrorString(e));
-    attr_set = true;
-  }
+  static MoeLdsOptIn opted;  // per instantiation
+  if (int rc = moe_opt_in_lds(opted, reinterpret_cast<const void*>(kern), lds, "fused_experts")) return rc;
   const int64_t tiles = static_cast<int64_t>(p.num_m_blocks) * p.num_n_tiles;
   const int64_t grid = (tiles + kXcds - 1) / kXcds * kXcds;
   if (grid > INT32_MAX) return moe_fail(MOE_ERR_ARG, "fused_experts: grid of %lld workgroups", static_cast<long long>(grid));
@@ -1543,17 +1565,11 @@ static bool big_16bit_ok(const GemmParams& p, bool gated, int block_size, int64_
 // p1.xcd_bounds must be set; `done` holds one zeroed counter per m-block.
 template <typename Mma>
 int launch_big_fused(GemmParams& p1, GemmParams& p2, int block_size, int64_t sorted_cap, int32_t* done,
-                     hipStream_t s) {
+                     int32_t* status, hipStream_t s) {
   constexpr int lds = kBigLdsTotal;
   auto kern = big_fused_kernel<Mma>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess)
-      return moe_fail(MOE_ERR_LAUNCH, "fused_experts: cannot reserve %d B of LDS: %s", lds, hipGetErrorString(e));
-    attr_set = true;
-  }
+  static MoeLdsOptIn opted;
+  if (int rc = moe_opt_in_lds(opted, reinterpret_cast<const void*>(kern), lds, "fused_experts")) return rc;
   for (GemmParams* q : {&p1, &p2}) {
     q->align_bs = block_size;
     q->m_major = 1;
@@ -1564,9 +1580,8 @@ int launch_big_fused(GemmParams& p1, GemmParams& p2, int block_size, int64_t sor
   const int cap_mb = big_plan_cap(sorted_cap);
   const int64_t grid = static_cast<int64_t>(cap_mb) * (p1.num_n_tiles + p2.num_n_tiles) * kXcds;
   if (grid > INT32_MAX) return moe_fail(MOE_ERR_ARG, "fused_experts: grid of %lld workgroups", static_cast<long long>(grid));
-  // a poll is about a microsecond: two seconds, far beyond any launch of this kernel
-  constexpr int kSpinLimit = 2000000;
-  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(kThreads), lds, s, p1, p2, done, cap_mb, kSpinLimit);
+  hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(kThreads), lds, s, p1, p2, done, cap_mb,
+                     g_wait_limit.load(std::memory_order_relaxed), status);
   return moe_check_launch("fused_experts (gate-up and down pass, one launch)");
 }
 
@@ -1671,11 +1686,17 @@ MOE_EXPORT int moe_fused_experts_plan_layout(int T, int H, int I, int E, int K, 
   return 1;
 }
 
-MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
+// Argument checks shared by moe_fused_experts and moe_fused_experts_status.  `cap` receives the
+// length of sorted_token_ids the call works with: numel + E * (block_size - 1), which no
+// alignment of T * K ids over E experts can exceed.  A longer buffer is accepted and its
+// surplus ignored: every region of the workspace is laid out from `cap`, never from the
+// caller's figure.
+static int check_fused_args(const MoeFusedExpertsArgs* a, int64_t* cap, int64_t* need_ws) {
   if (!a) return moe_fail(MOE_ERR_ARG, "fused_experts: null argument block");
-  if (a->T < 0 || a->H < 1 || a->I < 1 || a->E < 1 || a->K < 1)
-    return moe_fail(MOE_ERR_ARG, "fused_experts: bad sizes T=%d H=%d I=%d E=%d K=%d", a->T, a->H, a->I, a->E, a->K);
-  if (a->T == 0) return MOE_OK;
+  if (a->T < 0 || a->H < 1 || a->I < 1 || a->E < 1 || a->K < 1 || a->block_size < 1)
+    return moe_fail(MOE_ERR_ARG, "fused_experts: bad sizes T=%d H=%d I=%d E=%d K=%d block_size=%d", a->T, a->H, a->I,
+                    a->E, a->K, a->block_size);
+  if (a->T == 0) { *cap = 0; *need_ws = 0; return MOE_OK; }
   if (!a->x || !a->out || !a->w13 || !a->w2 || !a->topk_weights || !a->sorted_token_ids ||
       !a->expert_ids || !a->num_tokens_post_pad)
     return moe_fail(MOE_ERR_ARG, "fused_experts: null tensor pointer");
@@ -1704,17 +1725,62 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   if (a->sorted_cap < need_cap)
     return moe_fail(MOE_ERR_ARG, "fused_experts: sorted_token_ids holds %lld, needs %lld",
                     static_cast<long long>(a->sorted_cap), static_cast<long long>(need_cap));
-  const int64_t need_ws = moe_fused_experts_workspace_bytes(a->T, a->H, a->I, a->E, a->K, a->block_size,
-                                                            a->act_dtype, a->weight_dtype);
-  if (!a->workspace || a->workspace_bytes < need_ws)
+  *need_ws = moe_fused_experts_workspace_bytes(a->T, a->H, a->I, a->E, a->K, a->block_size, a->act_dtype,
+                                               a->weight_dtype);
+  if (!a->workspace || a->workspace_bytes < *need_ws)
     return moe_fail(MOE_ERR_WORKSPACE, "fused_experts: workspace %lld B, needs %lld B",
-                    static_cast<long long>(a->workspace_bytes), static_cast<long long>(need_ws));
+                    static_cast<long long>(a->workspace_bytes), static_cast<long long>(*need_ws));
   if (reinterpret_cast<uintptr_t>(a->workspace) & 255u)
     return moe_fail(MOE_ERR_WORKSPACE, "fused_experts: workspace must be 256-byte aligned");
+  *cap = need_cap;
+  return MOE_OK;
+}
+
+// Whether this call enqueues the two GEMM passes as one launch (16-bit dtypes, blocks that are
+// multiples of 256 slots, both passes requested, operands within the DMA kernels' 32-bit offsets).
+static bool uses_one_launch(const MoeFusedExpertsArgs* a, int64_t cap) {
+  if (a->block_size % kBigBM != 0 || a->act_dtype == MOE_F32 || a->weight_dtype == MOE_E4M3) return false;
+  const int passes = (a->passes & 7) ? a->passes : (a->passes | 7);
+  if ((passes & 3) != 3 || (passes & 8)) return false;
+  GemmParams p1{}, p2{};
+  p1.numel = p2.numel = static_cast<int>(static_cast<int64_t>(a->T) * a->K);
+  p1.top_k = p2.top_k = a->K;
+  p1.lda = a->H; p1.Kd = a->H; p1.N = a->I; p1.w_stride_n = a->w13_stride_n; p1.a_by_slot = 0;
+  p2.lda = a->I; p2.Kd = a->I; p2.N = a->H; p2.w_stride_n = a->w2_stride_n; p2.a_by_slot = 1;
+  return big_16bit_ok(p1, true, a->block_size, cap) && big_16bit_ok(p2, false, a->block_size, cap);
+}
+
+MOE_EXPORT int moe_fused_experts_set_wait_limit(int polls) {
+  return g_wait_limit.exchange(polls < 0 ? 0 : polls, std::memory_order_relaxed);
+}
+
+MOE_EXPORT int moe_fused_experts_status(const MoeFusedExpertsArgs* a) {
+  int64_t cap = 0, need_ws = 0;
+  if (int rc = check_fused_args(a, &cap, &need_ws)) return rc;
+  if (a->T == 0 || !uses_one_launch(a, cap)) return MOE_OK;
+  const int32_t* word = reinterpret_cast<const int32_t*>(static_cast<const char*>(a->workspace) + need_ws - 256) +
+                        kBigStatusWord;
+  int32_t expired = 0;
+  hipStream_t s = static_cast<hipStream_t>(a->stream);
+  hipError_t e = hipMemcpyAsync(&expired, word, sizeof(expired), hipMemcpyDeviceToHost, s);
+  if (e == hipSuccess) e = hipStreamSynchronize(s);
+  if (e != hipSuccess) return moe_fail(MOE_ERR_LAUNCH, "fused_experts_status: %s", hipGetErrorString(e));
+  if (expired != 0)
+    return moe_fail(MOE_ERR_HANDOFF, "fused_experts: %d down tiles gave up waiting for the gate-up tiles of their "
+                    "block and wrote NaN rows (one-launch form; passes bit 8 selects two launches)", expired);
+  return MOE_OK;
+}
+
+MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
+  int64_t cap = 0, need_ws = 0;
+  if (int rc0 = check_fused_args(a, &cap, &need_ws)) return rc0;
+  if (a->T == 0) return MOE_OK;
+  const bool fp8 = a->weight_dtype == MOE_E4M3;
+  const int64_t numel = static_cast<int64_t>(a->T) * a->K;
 
   hipStream_t s = static_cast<hipStream_t>(a->stream);
   const int64_t es = elem_size(a->act_dtype);
-  const int64_t rows = moe_align_up(a->sorted_cap, a->block_size);
+  const int64_t rows = moe_align_up(cap, a->block_size);
   char* inter = static_cast<char*>(a->workspace);
   char* c3 = inter + moe_align_up(rows * a->I * es, 256);
   char* xq = c3 + moe_align_up(numel * a->H * es, 256);                        // fp8 only from here on
@@ -1728,7 +1794,7 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.num_post_pad = a->num_tokens_post_pad;
   p.topk_w = a->topk_weights;
   p.numel = static_cast<int>(numel);
-  p.sorted_cap = a->sorted_cap;
+  p.sorted_cap = cap;
   p.top_k = a->K;
   p.alpha = a->swiglu_alpha;
   p.limit = a->swiglu_limit;
@@ -1739,11 +1805,11 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   if (a->block_size % kBigBM == 0 && a->act_dtype != MOE_F32) {
     // both passes walk the same m-blocks: one plan for the two launches
     int32_t* bounds = reinterpret_cast<int32_t*>(static_cast<char*>(a->workspace) + need_ws - 256);
-    const int num_done = static_cast<int>((a->sorted_cap + kBigBM - 1) / kBigBM);
+    const int num_done = static_cast<int>((cap + kBigBM - 1) / kBigBM);
     plan_done = bounds - moe_align_up(static_cast<int64_t>(num_done) * 4, 256) / 4;
     if (!(a->passes & 16)) {  // bit 16: moe_align_block_size_planned already left the plan here
       hipLaunchKernelGGL(big_plan_kernel, dim3(1), dim3(kPlanThreads), 0, s, a->sorted_token_ids,
-                         a->num_tokens_post_pad, static_cast<int>(numel), big_plan_cap(a->sorted_cap), bounds,
+                         a->num_tokens_post_pad, static_cast<int>(numel), big_plan_cap(cap), bounds,
                          plan_done, num_done);
       if (int rc0 = moe_check_launch("fused_experts (XCD ranges)")) return rc0;
     }
@@ -1764,9 +1830,10 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
     p2.bias = a->w2_bias; p2.bias_stride_e = a->H;
     p2.c = c3; p2.ldc = a->H; p2.Kd = a->I; p2.N = a->H; p2.a_by_slot = 1;
     p2.mul_weight = a->apply_router_weight_on_input ? 0 : 1;
-    if (big_16bit_ok(p, true, a->block_size, a->sorted_cap) && big_16bit_ok(p2, false, a->block_size, a->sorted_cap)) {
-      rc = a->act_dtype == MOE_BF16 ? launch_big_fused<MmaBF16>(p, p2, a->block_size, a->sorted_cap, plan_done, s)
-                                    : launch_big_fused<MmaF16>(p, p2, a->block_size, a->sorted_cap, plan_done, s);
+    if (big_16bit_ok(p, true, a->block_size, cap) && big_16bit_ok(p2, false, a->block_size, cap)) {
+      int32_t* status = const_cast<int32_t*>(plan_bounds) + kBigStatusWord;
+      rc = a->act_dtype == MOE_BF16 ? launch_big_fused<MmaBF16>(p, p2, a->block_size, cap, plan_done, status, s)
+                                    : launch_big_fused<MmaF16>(p, p2, a->block_size, cap, plan_done, status, s);
       if (rc) return rc;
       if (!(passes & 4)) return MOE_OK;
       return moe_sum(a->out, c3, a->T, a->K, a->H, a->act_dtype, a->stream);
@@ -1777,12 +1844,12 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
     rc = moe_quant_rows_e4m3(a->x, a->act_dtype, a->T, a->H, reinterpret_cast<uint8_t*>(xq), xs, a->stream);
     if (rc) return rc;
     p.a = xq; p.a_scale = xs; p.w_scale = a->w13_scale; p.w_scale_stride_e = 2LL * a->I;
-    rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaE4M3<ElemBF16>, true>(p, a->block_size, a->sorted_cap, s)
-                                  : launch_bm<MmaE4M3<ElemF16>, true>(p, a->block_size, a->sorted_cap, s);
+    rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaE4M3<ElemBF16>, true>(p, a->block_size, cap, s)
+                                  : launch_bm<MmaE4M3<ElemF16>, true>(p, a->block_size, cap, s);
   } else if (passes & 1) {
-    rc = a->act_dtype == MOE_BF16  ? launch_bm<MmaBF16, true>(p, a->block_size, a->sorted_cap, s)
-         : a->act_dtype == MOE_F16 ? launch_bm<MmaF16, true>(p, a->block_size, a->sorted_cap, s)
-                                   : launch_bm<MmaF32, true>(p, a->block_size, a->sorted_cap, s);
+    rc = a->act_dtype == MOE_BF16  ? launch_bm<MmaBF16, true>(p, a->block_size, cap, s)
+         : a->act_dtype == MOE_F16 ? launch_bm<MmaF16, true>(p, a->block_size, cap, s)
+                                   : launch_bm<MmaF32, true>(p, a->block_size, cap, s);
   }
   if (rc) return rc;
 
@@ -1795,15 +1862,15 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   if (fp8 && (passes & 2)) {
     // the activated intermediate is quantised per slot row the same way
     rc = moe_quant_slot_rows_e4m3(inter, a->act_dtype, rows, a->I, reinterpret_cast<uint8_t*>(iq), is,
-                                  a->sorted_token_ids, a->sorted_cap, static_cast<int>(numel), a->stream);
+                                  a->sorted_token_ids, cap, static_cast<int>(numel), a->stream);
     if (rc) return rc;
     p.a = iq; p.a_scale = is; p.w_scale = a->w2_scale; p.w_scale_stride_e = a->H;
-    rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaE4M3<ElemBF16>, false>(p, a->block_size, a->sorted_cap, s)
-                                  : launch_bm<MmaE4M3<ElemF16>, false>(p, a->block_size, a->sorted_cap, s);
+    rc = a->act_dtype == MOE_BF16 ? launch_bm<MmaE4M3<ElemBF16>, false>(p, a->block_size, cap, s)
+                                  : launch_bm<MmaE4M3<ElemF16>, false>(p, a->block_size, cap, s);
   } else if (passes & 2) {
-    rc = a->act_dtype == MOE_BF16  ? launch_bm<MmaBF16, false>(p, a->block_size, a->sorted_cap, s)
-         : a->act_dtype == MOE_F16 ? launch_bm<MmaF16, false>(p, a->block_size, a->sorted_cap, s)
-                                   : launch_bm<MmaF32, false>(p, a->block_size, a->sorted_cap, s);
+    rc = a->act_dtype == MOE_BF16  ? launch_bm<MmaBF16, false>(p, a->block_size, cap, s)
+         : a->act_dtype == MOE_F16 ? launch_bm<MmaF16, false>(p, a->block_size, cap, s)
+                                   : launch_bm<MmaF32, false>(p, a->block_size, cap, s);
   }
   if (rc) return rc;
 

@@ -23,7 +23,6 @@ struct Pow2Geom {
 };
 
 constexpr int kWavesPerBlock = 4;
-constexpr float kFltMin = 1.17549435e-38f;
 
 // Lane exchange for the order-independent reductions (max, argmax): partner at
 // distance M inside a row of TPR lanes.  Distances 1 and 2 are exact xor
@@ -86,10 +85,7 @@ __device__ __forceinline__ void route_row(float (&v)[Pow2Geom<E>::kVpt], int t, 
   for (int m = TPR / 2; m > 0; m /= 2) sum += __shfl_xor(sum, m, kWave);
   const float rinv = 1.f / sum;
 #pragma unroll
-  for (int i = 0; i < VPT; ++i) {
-    float p = v[i] * rinv;
-    v[i] = p < kFltMin ? 0.f : p;
-  }
+  for (int i = 0; i < VPT; ++i) v[i] = v[i] * rinv;  // subnormal probabilities are kept, as the reference keeps them
 
   // Up to kRegK winners stay in registers until the row is done (after the
   // all-reduce every lane of the row knows them): the renormalised weights are
@@ -352,7 +348,7 @@ __global__ __launch_bounds__(kWave* kGateWaves) void gate_topk_softmax_kernel(
 }
 
 template <typename El, int E>
-void launch_gate(const void* x, const void* wg, float* logits_out, float* w, int32_t* ids,
+int launch_gate(const void* x, const void* wg, float* logits_out, float* w, int32_t* ids,
                  int32_t* tei, int T, int H, int K, int renorm, hipStream_t s) {
   using S = typename El::S;
   const int blocks = (T + kGateTokens - 1) / kGateTokens;
@@ -360,33 +356,28 @@ void launch_gate(const void* x, const void* wg, float* logits_out, float* w, int
   if (blocks <= 256) {
     constexpr int lds = 7 * (E + kGateTokens) * kGateRowBytes;
     auto kern = gate_topk_softmax_kernel<El, E, 7>;
-    static bool attr_set = false;  // dynamic LDS above 64 KB must be opted into
-    if (!attr_set) {
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-      attr_set = true;
-    }
+    static MoeLdsOptIn opted;
+    if (int rc = moe_opt_in_lds(opted, reinterpret_cast<const void*>(kern), lds, "gate_topk_softmax")) return rc;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(kWave * kGateWaves), lds, s,
                        static_cast<const S*>(x), static_cast<const S*>(wg), logits_out, w, ids, tei, T, H, K, renorm);
   } else {
     constexpr int lds = 4 * (E + kGateTokens) * kGateRowBytes;
     auto kern = gate_topk_softmax_kernel<El, E, 4>;
-    static bool attr_set = false;
-    if (!attr_set) {
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-      attr_set = true;
-    }
+    static MoeLdsOptIn opted;
+    if (int rc = moe_opt_in_lds(opted, reinterpret_cast<const void*>(kern), lds, "gate_topk_softmax")) return rc;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(kWave * kGateWaves), lds, s,
                        static_cast<const S*>(x), static_cast<const S*>(wg), logits_out, w, ids, tei, T, H, K, renorm);
   }
+  return MOE_OK;
 }
 
 template <typename El>
 int launch_gate_e(const void* x, const void* wg, float* logits_out, float* w, int32_t* ids,
                   int32_t* tei, int T, int H, int E, int K, int renorm, hipStream_t s) {
   switch (E) {
-    case 32: launch_gate<El, 32>(x, wg, logits_out, w, ids, tei, T, H, K, renorm, s); break;
-    case 64: launch_gate<El, 64>(x, wg, logits_out, w, ids, tei, T, H, K, renorm, s); break;
-    case 128: launch_gate<El, 128>(x, wg, logits_out, w, ids, tei, T, H, K, renorm, s); break;
+    case 32: if (int rc = launch_gate<El, 32>(x, wg, logits_out, w, ids, tei, T, H, K, renorm, s)) return rc; break;
+    case 64: if (int rc = launch_gate<El, 64>(x, wg, logits_out, w, ids, tei, T, H, K, renorm, s)) return rc; break;
+    case 128: if (int rc = launch_gate<El, 128>(x, wg, logits_out, w, ids, tei, T, H, K, renorm, s)) return rc; break;
     default: return moe_fail(MOE_ERR_UNSUPPORTED, "gate_topk_softmax: num_experts %d (32, 64 or 128)", E);
   }
   return moe_check_launch("gate_topk_softmax");
@@ -429,8 +420,7 @@ __global__ __launch_bounds__(kWave* kWavesPerBlock) void topk_softmax_generic_ke
 #pragma unroll
   for (int j = 0; j < kGenericMaxPerLane; ++j) {
     const int c = lane + j * kWave;
-    float p = v[j] * rinv;
-    p = p < kFltMin ? 0.f : p;
+    const float p = v[j] * rinv;
     v[j] = c < E ? p : -20000.f;  // columns past E can never win
   }
 

@@ -5,12 +5,18 @@ defaults, assertions and return values) on top of libmoe_gfx950.so.
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional, Tuple
 
 import torch
 
 from . import _lib, ops
 from ._lib import MoeFusedExpertsArgs, check, lib, stream_ptr
+
+
+# MOE_CHECK_HANDOFF=1: after every chunk wait for the stream and raise if a bounded device-side
+# wait of the one-launch form expired (a debugging aid: it synchronises, so not under graph capture)
+_CHECK_HANDOFF = os.environ.get("MOE_CHECK_HANDOFF", "0") == "1"
 
 
 def cdiv(a: int, b: int) -> int:
@@ -59,14 +65,18 @@ def _plan_in_workspace(workspace: torch.Tensor, T: int, H: int, I: int, E: int, 
 
 def try_get_optimal_moe_config(w1_shape, w2_shape, top_k: int, dtype: Optional[str], M: int,
                                is_marlin: bool = False,
-                               block_shape: Optional[list] = None) -> dict:
+                               block_shape: Optional[list] = None,
+                               act_dtype: torch.dtype = torch.bfloat16) -> dict:
     """Role of nanovllm/layers/for_moe/fused_moe.py:354-390.  The reference looks
     up Triton tile tables per device name; the HIP kernels own their tiling, so
     the only entry that still matters to callers is BLOCK_SIZE_M, the block size
-    handed to moe_align_block_size."""
+    handed to moe_align_block_size.  ``act_dtype`` (not in the reference, whose
+    ``dtype`` string only names quantised forms) is the activation dtype: fp32
+    runs on other kernels than the 16-bit dtypes and has its own rule."""
     E = w2_shape[0]
-    weight_code = _lib.E4M3_CODE if dtype == "fp8_w8a8" else _lib.DTYPE_CODE[torch.bfloat16]
-    bm = lib().moe_preferred_block_size(M, E, top_k, _lib.DTYPE_CODE[torch.bfloat16], weight_code)
+    act_code = _lib.DTYPE_CODE[act_dtype]
+    weight_code = _lib.E4M3_CODE if dtype == "fp8_w8a8" else act_code
+    bm = lib().moe_preferred_block_size(M, E, top_k, act_code, weight_code)
     return {"BLOCK_SIZE_M": bm}
 
 
@@ -161,13 +171,14 @@ def launch_fused_experts(x: torch.Tensor, out: torch.Tensor, w1: torch.Tensor, w
                          block_size: int, activation: str = "silu",
                          apply_router_weight_on_input: bool = False,
                          weight_code: Optional[int] = None,
-                         workspace: Optional[torch.Tensor] = None, passes: int = 0) -> None:
+                         workspace: Optional[torch.Tensor] = None, passes: int = 0) -> MoeFusedExpertsArgs:
     """One call of the C entry point ``moe_fused_experts`` on already aligned
     tokens (the part of nanovllm/layers/for_moe/fused_moe.py:579-631 after
     moe_align_block_size).  ``workspace`` (uint8) is allocated when not given;
     ``passes`` selects single passes for profiling (1 gate-up, 2 down, 4
     combine, 0 = all; adding 8 keeps the two GEMM passes in separate launches
-    where the library would enqueue them as one)."""
+    where the library would enqueue them as one).  Returns the argument block
+    (what ``fused_experts_status`` takes)."""
     T, H = x.shape
     E, N, _ = w1.shape
     top_k = topk_weights.shape[1]
@@ -200,6 +211,23 @@ def launch_fused_experts(x: torch.Tensor, out: torch.Tensor, w1: torch.Tensor, w
         swiglu_alpha=1.702, swiglu_limit=7.0, passes=passes, stream=stream_ptr(x.device))
     with torch.cuda.device(x.device):
         check(L.moe_fused_experts(args))
+    args._keepalive = (workspace,)
+    return args
+
+
+def fused_experts_status(args: MoeFusedExpertsArgs) -> None:
+    """``moe_fused_experts_status`` for the argument block of the most recent
+    ``launch_fused_experts`` call on its workspace: waits for the stream and raises
+    ``RuntimeError`` when a down tile of the one-launch form gave up waiting for
+    its block's gate-up tiles (its rows of the result are NaN then).  No
+    counterpart in the reference."""
+    check(lib().moe_fused_experts_status(args))
+
+
+def set_wait_limit(polls: int) -> int:
+    """``moe_fused_experts_set_wait_limit``: polls a down tile of the one-launch
+    form waits before giving up (process-wide); returns the previous value."""
+    return lib().moe_fused_experts_set_wait_limit(int(polls))
 
 
 def quantize_expert_weights(w13: torch.Tensor, w2: torch.Tensor):
@@ -251,7 +279,6 @@ def fused_experts_impl(hidden_states: torch.Tensor,
     assert w1_zp is None and w2_zp is None and block_shape is None and expert_map is None
     if activation not in _lib.ACTIVATION_CODE:
         raise ValueError(f"Unsupported FusedMoe activation: {activation}")
-    _lib.require_gpu_tensor(hidden_states, "hidden_states")
 
     fp8 = w1.dtype in _FP8_DTYPES or (w1_scale is not None)
     if fp8:
@@ -278,11 +305,23 @@ def fused_experts_impl(hidden_states: torch.Tensor,
     assert w2.size(2) == N // 2 and w2.size(0) == E, "w2 must be [E, H, I] for w1 [E, 2I, H]"
     if global_num_experts == -1:
         global_num_experts = E
+    # without an expert map (rejected above) every expert is local
+    assert global_num_experts == E, "global_num_experts must equal the number of local experts (no expert parallelism)"
+    # Narrower than the reference's Triton kernel, which masks ragged K and N
+    # (for_moe/fused_moe.py:191-205,218-223): rows are moved in 16-byte chunks.
+    chunk = 16 if fp8 else 8
+    assert hidden_states.size(1) % chunk == 0 and (N // 2) % chunk == 0, \
+        f"hidden size and intermediate size must be multiples of {chunk}"
+    assert all(st % chunk == 0 for st in (w1.stride(0), w1.stride(1), w2.stride(0), w2.stride(1))), \
+        f"weight strides must be multiples of {chunk} elements"
+    assert all(t.data_ptr() % 16 == 0 for t in (hidden_states, w1, w2)), "tensors must be 16-byte aligned"
+    _lib.require_gpu_tensor(hidden_states, "hidden_states")
     top_k_num = topk_ids.size(1)
     CHUNK_SIZE: int = 64 * 1024
     M = min(num_tokens, CHUNK_SIZE)
     config_dtype = "fp8_w8a8" if fp8 else None
-    config = try_get_optimal_moe_config(w1.size(), w2.size(), top_k_num, config_dtype, M)
+    config = try_get_optimal_moe_config(w1.size(), w2.size(), top_k_num, config_dtype, M,
+                                        act_dtype=hidden_states.dtype)
 
     out_hidden_states = hidden_states if inplace else torch.empty_like(hidden_states)
     if topk_weights.dtype != torch.float32:
@@ -302,7 +341,7 @@ def fused_experts_impl(hidden_states: torch.Tensor,
             break
         if tokens_in_chunk < CHUNK_SIZE and chunk > 0:
             config = try_get_optimal_moe_config(w1.size(), w2.size(), top_k_num, config_dtype,
-                                                tokens_in_chunk)
+                                                tokens_in_chunk, act_dtype=hidden_states.dtype)
         bm = config["BLOCK_SIZE_M"]
         curr_ids = topk_ids[begin:end]
         curr_w = topk_weights[begin:end]
@@ -317,9 +356,12 @@ def fused_experts_impl(hidden_states: torch.Tensor,
                                       act_code, weight_code, curr_ids.numel())
         sorted_token_ids, expert_ids, num_tokens_post_padded = _align_block_size(
             curr_ids, bm, global_num_experts, plan)
-        launch_fused_experts(hidden_states[begin:end], out_hidden_states[begin:end], w1, w2,
-                             w1_bias, w2_bias, w1_scale, w2_scale, curr_w, sorted_token_ids,
-                             expert_ids, num_tokens_post_padded, bm, activation,
-                             apply_router_weight_on_input, weight_code=weight_code,
-                             workspace=workspace, passes=16 if plan is not None else 0)
+        args = launch_fused_experts(hidden_states[begin:end], out_hidden_states[begin:end], w1, w2,
+                                    w1_bias, w2_bias, w1_scale, w2_scale, curr_w, sorted_token_ids,
+                                    expert_ids, num_tokens_post_padded, bm, activation,
+                                    apply_router_weight_on_input, weight_code=weight_code,
+                                    workspace=workspace, passes=16 if plan is not None else 0)
+        if _CHECK_HANDOFF:
+            fused_experts_status(args)
     return out_hidden_states
+

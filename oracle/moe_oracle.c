@@ -26,7 +26,10 @@
  *     the reference tree (CUDA toolkit 12.8 libdevice).  This oracle defines
  *     its own fp32 exp (oracle_expf: Cody-Waite reduction + degree-6
  *     polynomial, every operation an IEEE fp32 operation or an fmaf), checked
- *     to <= 2 ulp against double-precision exp.  The *bits* of the weights
+ *     to <= 2 ulp against double-precision exp, subnormal results included:
+ *     the reference is built without flush-to-zero (setup.py:46-47), so
+ *     probabilities between 2^-149 and 2^-126 keep their value and their
+ *     rank, as they do here.  The *bits* of the weights
  *     are therefore "parity unpinned" against the reference; their values
  *     agree with a float64 softmax to ~1e-7 relative.
  *   - The fallback path (E not a power of two, or E > 256) uses cub
@@ -61,7 +64,7 @@ static inline uint32_t float_to_bits(float f) {
 ORACLE_API float oracle_expf(float x) {
   if (x != x) return x;
   if (x > 88.0f) return INFINITY;
-  if (x < -87.0f) return 0.0f; /* results below ~1.6e-38 are flushed to zero */
+  if (x < -104.0f) return 0.0f; /* below 2^-150: rounds to zero */
   float n = rintf(x * 1.44269504088896341f);
   float r = fmaf(n, -0.693359375f, x);         /* ln2 high part, 9 bits */
   r = fmaf(n, 2.12194440e-4f, r);              /* minus ln2 low part    */
@@ -75,8 +78,16 @@ ORACLE_API float oracle_expf(float x) {
   p = fmaf(p, r2, r);
   p = p + 1.0f;
   /* scale by 2^n through the exponent field; p in [0.70, 1.42], n in
-     [-126, 127] after the cut-offs above, so no overflow of the field. */
+     [-150, 127] after the cut-offs above.  A result that may be subnormal
+     (n <= -126) is scaled in two steps, p * 2^(n+64) through the field (exact)
+     and one IEEE multiplication by 2^-64, which rounds once: the reference is
+     built without flush-to-zero (setup.py:46-47, plain -O3), so CUDA's expf
+     returns subnormals down to about -103.97 and so does this one. */
   int32_t ni = (int32_t)n;
+  if (ni < -125) {
+    float t = bits_to_float(float_to_bits(p) + ((uint32_t)(ni + 64) << 23));
+    return t * 5.42101086242752217e-20f; /* 2^-64 */
+  }
   return bits_to_float(float_to_bits(p) + ((uint32_t)ni << 23));
 }
 
@@ -137,10 +148,7 @@ static void softmax_row_pow2(const float* x, float* p, int E) {
   }
   /* scale by the reciprocal (:297-303) */
   float rinv = 1.f / tsum[0];
-  for (int c = 0; c < E; ++c) {
-    float v = p[c] * rinv;
-    p[c] = v < 1.17549435e-38f ? 0.f : v; /* subnormal products flushed */
-  }
+  for (int c = 0; c < E; ++c) p[c] = p[c] * rinv; /* subnormal products are kept (:297-303) */
 }
 
 /* Fallback for any other E (:50-106): 64 strided partial results combined by
@@ -172,10 +180,7 @@ static void softmax_row_generic(const float* x, float* p, int E) {
     memcpy(part, nxt, sizeof(part));
   }
   float rinv = 1.f / part[0];
-  for (int c = 0; c < E; ++c) {
-    float v = p[c] * rinv;
-    p[c] = v < 1.17549435e-38f ? 0.f : v;
-  }
+  for (int c = 0; c < E; ++c) p[c] = p[c] * rinv;
 }
 
 /* Returns 0, or -1 on bad arguments.  `probs_or_null` (T*E floats) receives

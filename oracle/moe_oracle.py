@@ -17,9 +17,17 @@ Two layers:
   The reference does this arithmetic in Triton ``tl.dot`` (third-party, not in
   the reference tree, pinned only as ``triton>=3.0.0``) and ships no test or
   golden vector for it, so ``fused_experts_ref`` is pinned by the textbook
-  special cases exercised in ``tests/test_oracle.py`` (K=1 gated MLP, E=1 dense
-  MLP, linearity in the routed weights, permutation invariance) and is
-  otherwise "parity unpinned" against the reference's own bits.
+  special cases exercised in ``tests/test_oracle.py``: K=1 gated MLP, E=1 dense
+  MLP, linearity in the routed weights, permutation invariance; every branch
+  (both biases, gelu, swigluoai, routed weight on the input side, the top-k sum)
+  against torch's float64 ``linear`` / ``silu`` / ``gelu`` per expert; both
+  mirrored rounding modes step by step on a hand-sized case.  The *bits* of the
+  reference's result (Triton's accumulation order) stay "parity unpinned".
+* ``fused_experts_fp8_ref`` has no counterpart in the reference (it asserts the
+  scales None); it is pinned as a definition: step by step against torch's own
+  ``float8_e4m3fn`` cast and ``F.linear`` with non-uniform row and channel
+  scales, and against ``fused_experts_ref`` on losslessly quantisable tensors up
+  to the provable bound of the one re-quantisation.
 """
 from __future__ import annotations
 
@@ -180,6 +188,7 @@ def gelu_and_mul(x: torch.Tensor) -> torch.Tensor:
 # fp8 e4m3fn (OCP) helpers, explicit so the rounding is not a library's choice
 # --------------------------------------------------------------------------
 E4M3_MAX = 448.0
+E4M3_MIN_SCALE = 2.0 ** -100  # below it 1 / s would overflow for tiny non-zero rows
 
 
 def _e4m3_table() -> np.ndarray:
@@ -222,12 +231,12 @@ def dequant_e4m3(code: torch.Tensor) -> torch.Tensor:
 
 def quant_weight_per_channel(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """[E, N, K] -> (codes uint8 [E,N,K], scales f32 [E,N]) with
-    s[e,n] = amax_k |w[e,n,k]| / 448 (1.0 for an all-zero channel) and codes
+    s[e,n] = max(amax_k |w[e,n,k]| / 448, 2^-100) (1.0 for an all-zero channel) and codes
     e4m3(w * (1 / s)), every operation a rounded fp32 one (the reciprocal form
     of dynamic fp8 quantisers: one division per row, one product per element)."""
     wf = _cpu(w).float()
     amax = wf.abs().amax(dim=-1)
-    s = torch.where(amax > 0, amax / E4M3_MAX, torch.ones_like(amax))
+    s = torch.where(amax > 0, torch.clamp(amax / E4M3_MAX, min=E4M3_MIN_SCALE), torch.ones_like(amax))
     q = quant_e4m3(wf * (1.0 / s)[..., None])
     return q, s
 
@@ -237,7 +246,7 @@ def quant_act_per_token(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     codes e4m3(x * (1 / s)), as ``quant_weight_per_channel``."""
     xf = _cpu(x).float()
     amax = xf.abs().amax(dim=-1)
-    s = torch.where(amax > 0, amax / E4M3_MAX, torch.ones_like(amax))
+    s = torch.where(amax > 0, torch.clamp(amax / E4M3_MAX, min=E4M3_MIN_SCALE), torch.ones_like(amax))
     q = quant_e4m3(xf * (1.0 / s)[:, None])
     return q, s
 

@@ -26,16 +26,25 @@ def _close(got, want, rtol=RTOL, atol=ATOL):
     assert not bad.any(), f"{bad.sum().item()} of {bad.numel()} off; max abs err {(got - want).abs().max().item():.4g}"
 
 
-def _close_mirrored(got, ref_fn, **tol):
-    """Against the oracle that rounds where the kernels store.  The large-tile
-    kernel forms silu(gate) * up on its fp32 accumulators and rounds the
-    intermediate once (``mirror_rounding="fused"``); the other kernels round at
-    every store the reference has (``True``).  Which kernel ran is the library's
-    choice, so either agreement is accepted, at the same tight tolerance."""
-    try:
-        _close(got, ref_fn(True), **tol)
-    except AssertionError:
-        _close(got, ref_fn("fused"), **tol)
+def _mode(moe, T, E, K, H, dtype, fp8=False, bm=None, activation="silu"):
+    """The rounding definition of the kernel the library picks for this call.  The
+    large-tile kernel (alignment blocks that are multiples of 256 slots, reduction
+    length of the gate-up pass a multiple of its K tile: 64 elements of 16 bits, 128
+    of e4m3) forms silu(gate) * up on its fp32 accumulators and rounds the
+    intermediate once (``mirror_rounding="fused"``); every other kernel, and the
+    large-tile kernel with the other activations, rounds at every store the
+    reference has (``True``)."""
+    if bm is None:
+        bm = moe.fused_moe.try_get_optimal_moe_config(
+            (E, 0, H), (E, H, 0), K, "fp8_w8a8" if fp8 else None, min(T, 65536), act_dtype=dtype)["BLOCK_SIZE_M"]
+    large = bm % 256 == 0 and H % (128 if fp8 else 64) == 0 and dtype != torch.float32
+    return "fused" if large and activation == "silu" else True
+
+
+def _close_mirrored(got, ref_fn, mode, **tol):
+    """Against the oracle that rounds where the kernel that ran stores (``_mode``)."""
+    assert mode is True or mode == "fused"
+    _close(got, ref_fn(mode), **tol)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -53,7 +62,7 @@ def test_fused_experts_against_oracle(moe, oracle, dev, dtype, E, H, I, T, K):
     # against the oracle that rounds where the reference stores intermediates the
     # agreement is much tighter (only the fp32 summation order differs)
     _close_mirrored(out, lambda m: oracle.fused_experts_ref(x, w13, w2, tw, ids, mirror_rounding=m),
-                    rtol=1.6e-2, atol=2e-3)
+                    _mode(moe, T, E, K, H, dtype), rtol=1.6e-2, atol=2e-3)
 
 
 @pytest.mark.parametrize("E,H,I,T,K", [(8, 256, 128, 64, 2), (16, 512, 192, 300, 4), (3, 72, 40, 50, 2)])
@@ -102,7 +111,8 @@ def test_bias_router_weight_on_input_and_other_activations(moe, oracle, dev):
                                     apply_router_weight_on_input=on_input)
             _close_mirrored(out, lambda m: oracle.fused_experts_ref(
                 x, w13, w2, tw, ids, activation=act, w1_bias=b13, w2_bias=b2,
-                apply_router_weight_on_input=on_input, mirror_rounding=m), rtol=2e-2, atol=4e-3)
+                apply_router_weight_on_input=on_input, mirror_rounding=m),
+                _mode(moe, T, E, K, H, torch.bfloat16, activation=act), rtol=2e-2, atol=4e-3)
     with pytest.raises(ValueError, match="Unsupported FusedMoe activation"):
         moe.fused_experts(d(x), d(w13), d(w2), None, None, d(tw), d(ids), activation="relu")
 
@@ -121,6 +131,8 @@ def test_strided_expert_weights(moe, oracle, dev):
 
 
 def test_linearity_and_permutation_properties_at_full_decode_size(moe, oracle, dev):
+    """Config 2 (256 decode tokens): every row against the fp32 oracle and against the
+    oracle that rounds where the kernel stores, plus the size-independent properties."""
     wl = moe.workloads
     shape, x, logits, w13, w2 = wl.make_config("decode_256")
     d = lambda t: t.to(dev)
@@ -132,15 +144,16 @@ def test_linearity_and_permutation_properties_at_full_decode_size(moe, oracle, d
     _close(b, a[perm].cpu(), rtol=1e-2, atol=2e-3)
     z = moe.fused_experts(d(x), d(w13), d(w2), None, None, torch.zeros_like(tw), ids)
     assert torch.count_nonzero(z) == 0
-    # sampled rows against the fp32 oracle
-    rows = torch.arange(0, x.shape[0], 8)
-    ref = oracle.fused_experts_ref(x[rows], w13, w2, tw.cpu()[rows], ids.cpu()[rows])
-    _close(a[rows.to(dev)], ref)
+    _close(a, oracle.fused_experts_ref(x, w13, w2, tw.cpu(), ids.cpu()))
+    mode = _mode(moe, x.shape[0], shape.experts, shape.top_k, shape.hidden, torch.bfloat16)
+    _close(a, oracle.fused_experts_ref(x, w13, w2, tw.cpu(), ids.cpu(), mirror_rounding=mode), rtol=1.6e-2, atol=2e-3)
 
 
-def test_layered_prefill_batch_sampled_rows(moe, oracle, dev):
-    """Config 3 (8192 prefill + 256 decode tokens): every row is independent of
-    the others, so a sample of rows is checked against the fp32 oracle."""
+def test_layered_prefill_batch_every_row(moe, oracle, dev):
+    """Config 3 (8192 prefill + 256 decode tokens): all 8448 rows against the fp32
+    oracle at the north-star tolerance and, tightly, against the oracle that rounds
+    where the large-tile kernel stores.  Config 4: each of the 16 chunks (512 prefill
+    rows + the 256 decode rows) gives the rows of the single pass."""
     wl = moe.workloads
     shape, x, logits, w13, w2 = wl.make_config("layered_8192p_256d")
     d = lambda t: t.to(dev)
@@ -148,16 +161,17 @@ def test_layered_prefill_batch_sampled_rows(moe, oracle, dev):
     tw, ids, _ = moe.fused_topk(d(x), d(logits), shape.top_k, True)
     out = moe.fused_experts(d(x), w13d, w2d, None, None, tw, ids)
     torch.cuda.synchronize()
-    rows = torch.cat([torch.arange(0, 8192, 257), torch.arange(8192, 8448, 31)])
-    ref = oracle.fused_experts_ref(x[rows], w13, w2, tw.cpu()[rows], ids.cpu()[rows])
-    _close(out[rows.to(dev)], ref)
+    _close(out, oracle.fused_experts_ref(x, w13, w2, tw.cpu(), ids.cpu()))
+    mode = _mode(moe, x.shape[0], shape.experts, shape.top_k, shape.hidden, torch.bfloat16)
+    assert mode == "fused"
+    _close(out, oracle.fused_experts_ref(x, w13, w2, tw.cpu(), ids.cpu(), mirror_rounding=mode), rtol=1.6e-2, atol=2e-3)
     # chunked prefill (16 x (512 + 256)) gives the same rows as the single pass
-    dec = slice(8192, 8448)
-    for c in (0, 7, 15):
+    outc = out.cpu()
+    for c in range(16):
         sel = torch.cat([torch.arange(c * 512, (c + 1) * 512), torch.arange(8192, 8448)]).to(dev)
         part = moe.fused_experts(d(x)[sel].contiguous(), w13d, w2d, None, None, tw[sel].contiguous(),
                                  ids[sel].contiguous())
-        _close(part, out[sel].cpu(), rtol=1e-2, atol=2e-3)
+        _close(part, outc[sel.cpu()], rtol=1e-2, atol=2e-3)
 
 
 def test_fused_moe_module_forward(moe, oracle, dev):
@@ -211,12 +225,17 @@ def test_moe_sum(moe, dev, dtype):
 def test_quant_rows_e4m3_matches_oracle(moe, oracle, dev):
     w = torch.randn(64, 512, generator=torch.Generator().manual_seed(7)) * 0.02
     w[3] = 0
+    w[5] = 0
+    w[5, 9], w[5, 200] = 1e-38, -3e-39          # 1 / (amax / 448) would overflow: the scale is floored
+    w[6] *= 2.0 ** -95                           # rows around the floor of 2^-100
+    w[7] *= 2.0 ** -105
     for dtype in (torch.float32, torch.bfloat16):
         wd = w.to(dtype)
         q, s = moe.ops.quant_rows_e4m3(wd.to(dev))
         oq, os_ = oracle.quant_weight_per_channel(wd[None])
         assert torch.equal(s.cpu(), os_[0])
         assert torch.equal(q.cpu(), oq[0])
+        assert not ((q.cpu() & 0x7f) == 0x7f).any() and s.cpu()[5] == 2.0 ** -100
 
 
 # ------------------------------------------------------------------ fp8 e4m3 variant
@@ -243,7 +262,8 @@ def test_fused_experts_fp8_against_dequantised_oracle(moe, oracle, dev, E, H, I,
     assert out.dtype == torch.bfloat16
     # (a) the oracle that rounds where the kernels store 16-bit intermediates: tight
     _close_mirrored(out, lambda m: oracle.fused_experts_fp8_ref(x, oq13, os13, oq2, os2, tw, ids, mirror_rounding=m),
-                    rtol=2e-2, atol=0.03 * out.float().abs().max().item())
+                    _mode(moe, T, E, K, H, torch.bfloat16, fp8=True), rtol=2e-2,
+                    atol=0.03 * out.float().abs().max().item())
     # (b) the pure fp32 dequantised oracle.  These small layers use 2.5x larger weights
     # than the benchmark layer, so the absolute floor is stated relative to the output
     # scale: one e4m3 step (2^-3 relative) of a typical element.  Re-quantising the
@@ -272,12 +292,14 @@ def test_fp8_every_block_size_kernel(moe, oracle, dev, bm, dtype, monkeypatch):
     torch.cuda.synchronize()
     _close_mirrored(out, lambda m: oracle.fused_experts_fp8_ref(
         x, w13q.view(torch.uint8).cpu(), w13s.cpu(), w2q.view(torch.uint8).cpu(), w2s.cpu(), tw, ids,
-        mirror_rounding=m), rtol=2e-2, atol=0.03 * out.float().abs().max().item())
+        mirror_rounding=m), _mode(moe, 700, 16, 4, 512, dtype, fp8=True, bm=bm), rtol=2e-2,
+        atol=0.03 * out.float().abs().max().item())
 
 
-def test_fp8_layered_prefill_batch_sampled_rows(moe, oracle, dev):
+def test_fp8_layered_prefill_batch_every_eighth_row(moe, oracle, dev):
     """Config 5: the 8192+256 batch with e4m3 weights and per-token e4m3
-    activations; sampled rows against the fp32 dequantised oracle."""
+    activations, against the fp32 dequantised oracle and the one that rounds where the
+    kernels store."""
     wl = moe.workloads
     shape, x, logits, w13, w2 = wl.make_config("layered_8192p_256d")
     d = lambda t: t.to(dev)
@@ -286,10 +308,17 @@ def test_fp8_layered_prefill_batch_sampled_rows(moe, oracle, dev):
     out = moe.fused_experts(d(x), w13q, w2q, None, None, tw, ids, per_channel_quant=True,
                             w1_scale=w13s, w2_scale=w2s)
     torch.cuda.synchronize()
-    rows = torch.cat([torch.arange(0, 8192, 513), torch.arange(8192, 8448, 63)])
-    ref = oracle.fused_experts_fp8_ref(x[rows], w13q.view(torch.uint8).cpu(), w13s.cpu(),
-                                       w2q.view(torch.uint8).cpu(), w2s.cpu(), tw.cpu()[rows], ids.cpu()[rows])
+    # every eighth prefill row and every decode row (1280 rows; the e4m3 oracle dequantises
+    # every expert's weights through a table, which is what bounds the sample)
+    rows = torch.cat([torch.arange(0, 8192, 8), torch.arange(8192, 8448)])
+    q13, q2 = w13q.view(torch.uint8).cpu(), w2q.view(torch.uint8).cpu()
+    ref = oracle.fused_experts_fp8_ref(x[rows], q13, w13s.cpu(), q2, w2s.cpu(), tw.cpu()[rows], ids.cpu()[rows])
     _close_fp8(out[rows.to(dev)], ref)
+    mode = _mode(moe, x.shape[0], shape.experts, shape.top_k, shape.hidden, torch.bfloat16, fp8=True)
+    assert mode == "fused"
+    refm = oracle.fused_experts_fp8_ref(x[rows], q13, w13s.cpu(), q2, w2s.cpu(), tw.cpu()[rows], ids.cpu()[rows],
+                                        mirror_rounding=mode)
+    _close(out[rows.to(dev)], refm, rtol=3e-2, atol=0.04 * out.float().abs().max().item())
 
 
 def test_layer_step_replays_from_a_hip_graph(moe, oracle, dev):
@@ -368,11 +397,13 @@ def test_random_shapes_all_kernels(moe, oracle, dev, case, monkeypatch):
         # tie) moves that term by 6 %: the bound stays inside the 6e-2 the fp8 path is held to
         _close_mirrored(out, lambda m: oracle.fused_experts_fp8_ref(
             x, w13q.view(torch.uint8).cpu(), w13s.cpu(), w2q.view(torch.uint8).cpu(), w2s.cpu(), tw, ids,
-            mirror_rounding=m), rtol=3e-2, atol=0.04 * out.float().abs().max().item() + 1e-6)
+            mirror_rounding=m), _mode(moe, T, E, K, H, dtype, fp8=True, bm=bm or None), rtol=3e-2,
+            atol=0.04 * out.float().abs().max().item() + 1e-6)
     else:
         out = moe.fused_experts(d(x), d(w13), d(w2), None, None, d(tw), d(ids))
         _close_mirrored(out, lambda m: oracle.fused_experts_ref(x, w13, w2, tw, ids, mirror_rounding=m),
-                        rtol=1.6e-2, atol=2e-3 + 4e-3 * out.float().abs().max().item())
+                        _mode(moe, T, E, K, H, dtype, bm=bm or None), rtol=1.6e-2,
+                        atol=2e-3 + 4e-3 * out.float().abs().max().item())
 
 
 @pytest.mark.gpu
@@ -433,7 +464,7 @@ def test_large_tile_ranges_on_lopsided_routing(moe, oracle, dev, pattern, monkey
     d = lambda t: t.to(dev)
     out = moe.fused_experts(d(x), d(w13), d(w2), None, None, d(tw), d(ids))
     _close_mirrored(out, lambda m: oracle.fused_experts_ref(x, w13, w2, tw, ids, mirror_rounding=m),
-                    rtol=1.6e-2, atol=2e-3 + 4e-3 * out.float().abs().max().item())
+                    "fused", rtol=1.6e-2, atol=2e-3 + 4e-3 * out.float().abs().max().item())
 
 
 @pytest.mark.gpu
@@ -520,3 +551,70 @@ def test_one_launch_form_on_two_streams(moe, oracle, dev):
     torch.cuda.synchronize()
     for j in jobs:
         assert torch.equal(j["out"], j["alone"])
+
+
+@pytest.mark.gpu
+def test_expired_wait_of_the_one_launch_form_is_reported(moe, oracle, dev):
+    """The down tiles of the one-launch form wait, boundedly, for their block's gate-up
+    tiles.  With the wait limit forced to 0 from the host every down tile that finds its
+    block incomplete gives up at once (here: all 24 tiles of an XCD start together, so the
+    down tiles do meet unfinished blocks).  Such a tile must not multiply a partly written
+    intermediate: it writes NaN rows, the status call reports it, every kernel exits
+    normally, and the next call with the default limit is clean again."""
+    fm = moe.fused_moe
+    E, H, I, T, K = 16, 512, 256, 2500, 4
+    x, w13, w2, logits = _layer(E, H, I, T, K, 300 + E, torch.bfloat16)
+    tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
+    d = lambda t: t.to(dev)
+    x, w13, w2, tw, ids = d(x), d(w13), d(w2), d(tw), d(ids)
+    so, eo, npp = fm.moe_align_block_size(ids, 256, E)
+    ws = torch.empty(fm.fused_experts_workspace_bytes(T, H, I, E, K, 256, torch.bfloat16), dtype=torch.uint8, device=dev)
+    good = torch.empty_like(x)
+    args = fm.launch_fused_experts(x, good, w13, w2, None, None, None, None, tw, so, eo, npp, 256, workspace=ws)
+    fm.fused_experts_status(args)                       # default limit: nothing expired
+    assert not torch.isnan(good).any()
+    old = fm.set_wait_limit(0)
+    try:
+        bad = torch.empty_like(x)
+        args = fm.launch_fused_experts(x, bad, w13, w2, None, None, None, None, tw, so, eo, npp, 256, workspace=ws)
+        with pytest.raises(RuntimeError, match="gave up waiting"):
+            fm.fused_experts_status(args)
+        torch.cuda.synchronize()                         # the launch has drained
+        nan_rows = torch.isnan(bad).any(dim=1)
+        assert nan_rows.any()
+        # rows no expired tile touched are the good ones, bit for bit
+        clean = ~torch.isnan(bad)
+        assert torch.equal(bad[clean], good[clean])
+    finally:
+        assert fm.set_wait_limit(old) == 0
+    again = torch.empty_like(x)
+    args = fm.launch_fused_experts(x, again, w13, w2, None, None, None, None, tw, so, eo, npp, 256, workspace=ws)
+    fm.fused_experts_status(args)
+    assert torch.equal(again, good)
+    # two launches (passes bit 8) have no hand-off: the status call has nothing to read
+    args = fm.launch_fused_experts(x, again, w13, w2, None, None, None, None, tw, so, eo, npp, 256, workspace=ws,
+                                   passes=7 | 8)
+    fm.fused_experts_status(args)
+
+
+@pytest.mark.gpu
+def test_longer_sorted_ids_buffer_is_accepted_and_its_surplus_ignored(moe, oracle, dev):
+    """A C caller may hand over a sorted_token_ids buffer longer than T*K + E*(block-1): the
+    workspace layout must not follow the caller's figure (it once did, and the regions
+    overlapped).  Same result as with the exact length."""
+    fm = moe.fused_moe
+    E, H, I, T, K = 8, 256, 128, 1200, 2
+    x, w13, w2, logits = _layer(E, H, I, T, K, 55, torch.bfloat16)
+    tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
+    d = lambda t: t.to(dev)
+    x, w13, w2, tw, ids = d(x), d(w13), d(w2), d(tw), d(ids)
+    for bs in (256, 32):
+        so, eo, npp = fm.moe_align_block_size(ids, bs, E)
+        exact = torch.empty_like(x)
+        fm.launch_fused_experts(x, exact, w13, w2, None, None, None, None, tw, so, eo, npp, bs)
+        longer = torch.cat([so, torch.full((5000,), T * K, dtype=torch.int32, device=dev)])
+        out = torch.empty_like(x)
+        fm.launch_fused_experts(x, out, w13, w2, None, None, None, None, tw, longer, eo, npp, bs)
+        torch.cuda.synchronize()
+        assert torch.equal(out, exact)
+        _close(out, oracle.fused_experts_ref(x.cpu(), w13.cpu(), w2.cpu(), tw.cpu(), ids.cpu()))

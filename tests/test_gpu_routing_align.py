@@ -50,6 +50,27 @@ def test_topk_softmax_extreme_logits(moe, oracle, dev):
     assert torch.equal(ids, oids) and torch.equal(w.view(torch.int32), ow.view(torch.int32))
 
 
+@pytest.mark.parametrize("E", [8, 128, 100])
+def test_topk_softmax_subnormal_probabilities_keep_their_rank(moe, oracle, dev, E):
+    """Logits 87 to 104 below the row maximum: the reference (built without
+    flush-to-zero) ranks their subnormal probabilities by value; below that they are
+    exactly zero and the lowest index wins.  Ids and weight bits as the oracle."""
+    g = torch.Generator().manual_seed(40 + E)
+    T = 96
+    x = -(torch.rand(T, E, generator=g) * 40 + 80)         # spread 80 .. 120 below the maximum
+    x[torch.arange(T), torch.randint(0, E, (T,), generator=g)] = 0.0
+    x[0] = torch.tensor([0.0, -95.0, -101.0, -90.0, -130.0, -99.0, -110.0, -120.0]).repeat(E // 8 + 1)[:E]
+    K = min(8, E)
+    for renorm in (False, True):
+        w, ids, tei = _run_topk(moe, x, K, renorm, dev)
+        ow, oids, otei, probs = oracle.topk_softmax(x, K, renormalize=renorm, return_probs=True)
+        assert torch.equal(ids, oids), renorm
+        assert torch.equal(w.view(torch.int32), ow.view(torch.int32)), renorm
+    sub = (probs > 0) & (probs < 2.0 ** -126)
+    assert sub.sum() > T                                      # the regime is exercised
+    assert ((ow > 0) & (ow < 2.0 ** -126)).any() or renorm    # and reaches the selected weights
+
+
 def test_fused_topk_matches_oracle_at_full_size(moe, oracle, dev):
     shape, x, logits, _, _ = None, None, None, None, None
     wl = moe.workloads

@@ -136,6 +136,68 @@ def test_fused_experts_shape_assertions(moe):
         moe.fused_experts(x, w1, w2, None, None, tw, ids, activation="relu")
 
 
+def test_fused_experts_states_its_narrower_contract(moe):
+    """The reference's Triton kernel masks ragged K and N (for_moe/fused_moe.py:191-205,218-223);
+    this build moves rows in 16-byte chunks and says so where the reference asserts."""
+    tw = torch.zeros(4, 2)
+    ids = torch.zeros(4, 2, dtype=torch.int32)
+    x = torch.zeros(4, 60, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError, match="multiples of 8"):
+        moe.fused_experts(x, torch.zeros(2, 32, 60, dtype=torch.bfloat16), torch.zeros(2, 60, 16, dtype=torch.bfloat16),
+                          None, None, tw, ids)
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError, match="multiples of 8"):
+        moe.fused_experts(x, torch.zeros(2, 24, 64, dtype=torch.bfloat16), torch.zeros(2, 64, 12, dtype=torch.bfloat16),
+                          None, None, tw, ids)
+    w1 = torch.zeros(2, 32, 68, dtype=torch.bfloat16)[:, :, :64]      # row stride 68
+    with pytest.raises(AssertionError, match="weight strides"):
+        moe.fused_experts(x, w1, torch.zeros(2, 64, 16, dtype=torch.bfloat16), None, None, tw, ids)
+    with pytest.raises(AssertionError, match="global_num_experts"):
+        moe.fused_experts(x, torch.zeros(2, 32, 64, dtype=torch.bfloat16), torch.zeros(2, 64, 16, dtype=torch.bfloat16),
+                          None, None, tw, ids, global_num_experts=4)
+    with pytest.raises(RuntimeError, match="no CPU path"):           # and only then the device check
+        moe.fused_experts(x, torch.zeros(2, 32, 64, dtype=torch.bfloat16), torch.zeros(2, 64, 16, dtype=torch.bfloat16),
+                          None, None, tw, ids)
+
+
+def test_block_size_rule_follows_the_activation_dtype(moe):
+    cfg = moe.fused_moe.try_get_optimal_moe_config
+    w1, w2 = (128, 1536, 2048), (128, 2048, 768)
+    assert cfg(w1, w2, 8, None, 768, act_dtype=torch.bfloat16)["BLOCK_SIZE_M"] == 256
+    assert cfg(w1, w2, 8, None, 768, act_dtype=torch.float16)["BLOCK_SIZE_M"] == 256
+    assert cfg(w1, w2, 8, None, 768, act_dtype=torch.float32)["BLOCK_SIZE_M"] == 64    # fp32 has its own rule
+    assert cfg(w1, w2, 8, None, 2048, act_dtype=torch.float32)["BLOCK_SIZE_M"] == 128
+    assert cfg(w1, w2, 8, "fp8_w8a8", 384)["BLOCK_SIZE_M"] == 32
+
+
+def test_plan_and_counters_lie_inside_the_workspace_behind_the_data(moe):
+    """Every region of a moe_fused_experts workspace is laid out from
+    T*K + E*(block-1), never from the length of the caller's sorted_token_ids buffer:
+    the per-block counters and the range table sit behind the intermediates."""
+    L = moe._lib.lib()
+    for T, H, I, E, K, bs, act, wgt in ((8448, 2048, 768, 128, 8, 256, 2, 2), (256, 2048, 768, 128, 8, 256, 2, 2),
+                                        (1, 64, 64, 4, 1, 256, 1, 1), (3000, 512, 256, 16, 4, 512, 2, 3),
+                                        (777, 128, 96, 8, 2, 256, 2, 3)):
+        total = L.moe_fused_experts_workspace_bytes(T, H, I, E, K, bs, act, wgt)
+        b, d = ctypes.c_int64(), ctypes.c_int64()
+        n, cap = ctypes.c_int32(), ctypes.c_int32()
+        assert L.moe_fused_experts_plan_layout(T, H, I, E, K, bs, act, wgt, ctypes.byref(b), ctypes.byref(d),
+                                               ctypes.byref(n), ctypes.byref(cap)) == 1
+        sorted_cap = T * K + E * (bs - 1)
+        rows = -(-sorted_cap // bs) * bs
+        up = lambda v: -(-v // 256) * 256
+        data = up(rows * I * 2) + up(T * K * H * 2)
+        if wgt == 3:
+            data += up(T * H) + up(T * 4) + up(rows * I) + up(rows * 4)
+        assert n.value == -(-sorted_cap // 256) and 1 <= cap.value <= n.value
+        assert d.value >= data and d.value + 4 * n.value <= b.value and b.value + 256 == total
+    # blocks that are not multiples of 256, or fp32, have no plan
+    assert L.moe_fused_experts_plan_layout(256, 2048, 768, 128, 8, 32, 2, 2, ctypes.byref(b), ctypes.byref(d),
+                                           ctypes.byref(n), ctypes.byref(cap)) == 0
+    assert L.moe_fused_experts_plan_layout(256, 2048, 768, 128, 8, 256, 0, 0, ctypes.byref(b), ctypes.byref(d),
+                                           ctypes.byref(n), ctypes.byref(cap)) == 0
+
+
 def test_workloads_are_reproducible_and_skewed(moe):
     wl = moe.workloads
     a = wl.make_inputs(wl.QWEN3_30B_A3B, 256, 1, torch.bfloat16)

@@ -20,10 +20,45 @@ def test_expf_within_2ulp_of_float64(oracle):
 
 
 def test_expf_special_values(oracle):
-    x = torch.tensor([0.0, -100.0, -87.5, 89.0, float("inf"), float("-inf"), float("nan")])
+    x = torch.tensor([0.0, -105.0, -200.0, 89.0, float("inf"), float("-inf"), float("nan")])
     y = oracle.expf(x)
     assert y[0] == 1.0 and y[1] == 0.0 and y[2] == 0.0
     assert math.isinf(y[3]) and math.isinf(y[4]) and y[5] == 0.0 and math.isnan(y[6])
+
+
+def test_expf_returns_subnormals_like_an_unflushed_expf(oracle):
+    """The reference is compiled without flush-to-zero (setup.py:46-47 passes plain
+    -O3 to nvcc), so its expf returns subnormal results for inputs between about
+    -87.34 and -103.97 and its router orders experts by them.  The oracle's exp
+    does the same: within 2 units of the subnormal spacing (2^-149) of float64
+    exp, monotone, non-zero down to ln(2^-149), zero below ln(2^-150)."""
+    x = torch.linspace(-104.0, -87.0, 170001).float()
+    y = oracle.expf(x).double().numpy()
+    ref = np.exp(x.double().numpy())
+    ulp = np.maximum(np.spacing(ref.astype(np.float32)).astype(np.float64), 2.0 ** -149)
+    assert (np.abs(y - ref) / ulp).max() <= 2.0
+    assert (np.diff(y) >= 0).all()
+    tiny = 2.0 ** -126
+    assert ((y > 0) & (y < tiny)).sum() > 100000          # subnormal results exist and are kept
+    assert oracle.expf(torch.tensor([-103.0]))[0] == 2.0 ** -149 * round(math.exp(-103.0) / 2.0 ** -149)
+    assert oracle.expf(torch.tensor([-103.2]))[0] > 0 and oracle.expf(torch.tensor([-104.0]))[0] == 0
+
+
+def test_routing_orders_experts_by_subnormal_probabilities(oracle):
+    """Logits 87 to 104 below the row maximum have subnormal probabilities: the
+    reference (no flush-to-zero) still ranks them by value, and only below that,
+    where they are exactly zero, does the lowest index win."""
+    row = torch.tensor([[-120.0, -95.0, 0.0, -101.0, -90.0, -130.0, -99.0, -110.0]])
+    w, ids, _, probs = oracle.topk_softmax(row, 8, return_probs=True)
+    assert ids[0].tolist() == [2, 4, 1, 6, 3, 0, 5, 7]
+    p = probs[0].double()
+    assert 0 < p[3] < p[6] < p[1] < p[4] < 2.0 ** -126     # subnormal, ordered by value
+    assert p[0] == 0 and p[5] == 0 and p[7] == 0          # below 2^-150: ties, lowest index first
+    want = torch.softmax(row.double(), -1)[0]
+    assert ((p - want).abs() <= 2.0 ** -148).all()
+    # a flush-to-zero build would return [2, 4?, ...] with experts 1, 3, 6 tied at zero: ids 0, 1, 3 ...
+    flushed = torch.where(p < 2.0 ** -126, torch.zeros_like(p), p)
+    assert torch.argsort(flushed, descending=True, stable=True).tolist() != ids[0].tolist()
 
 
 def test_expf_is_monotone_on_softmax_range(oracle):
@@ -402,3 +437,284 @@ def test_add_rms_norm_known_answers(oracle):
     assert torch.equal(new_res, s64.to(torch.bfloat16))
     want = new_res.double() / torch.sqrt((s64 * s64).mean(-1, keepdim=True) + 1e-6) * w.double()
     assert ((out.double() - want).abs() <= 2.0 ** -7 * want.abs() + 1e-12).all()
+
+
+# ----------------------------------------------------------------- expert MLP: every branch
+def _mlp64(x, w13, w2, act, b13=None, b2=None, in_weight=None, out_weight=None):
+    """One expert's gated MLP written with torch library routines in float64:
+    the textbook form the branches of ``fused_experts_ref`` are pinned to
+    (nanovllm/layers/for_moe/fused_moe.py:207-214 bias then routed weight;
+    csrc/activation_kernels.cu:8-64; moe_easy_kernel.py:89-98)."""
+    F = torch.nn.functional
+    h = F.linear(x.double(), w13.double(), None if b13 is None else b13.double())
+    if in_weight is not None:
+        h = h * in_weight.double()[:, None]           # weight multiplies sum + bias
+    I = w2.shape[-1]
+    if act == "silu":
+        a = F.silu(h[:, :I]) * h[:, I:]
+    elif act == "gelu":
+        a = F.gelu(h[:, :I]) * h[:, I:]                # erf form, gate = first half
+    else:                                              # swigluoai: gate/up interleaved, clamped
+        g, u = h[:, 0::2].clamp(max=7.0), h[:, 1::2].clamp(-7.0, 7.0)
+        a = (u + 1.0) * g * torch.sigmoid(1.702 * g)
+    o = F.linear(a, w2.double(), None if b2 is None else b2.double())
+    if out_weight is not None:
+        o = o * out_weight.double()[:, None]
+    return o
+
+
+@pytest.mark.parametrize("act", ["silu", "gelu", "swigluoai"])
+@pytest.mark.parametrize("on_input", [False, True])
+@pytest.mark.parametrize("bias", [False, True])
+def test_fused_experts_branches_against_library_mlp(oracle, act, on_input, bias):
+    """K=1 per token, several experts: each token's row must be the float64 library
+    MLP of its expert, with the bias added before the routed weight multiplies and
+    the weight applied on the chosen side.  A swapped gate/up half, a bias added
+    after the weight, tanh instead of erf GELU, a missing clamp or de-interleave,
+    or the weight applied on both / neither side each fail this."""
+    E, H, I, T = 3, 48, 40, 29
+    g = torch.Generator().manual_seed(100 + len(act) + 2 * on_input + bias)
+    x = torch.randn(T, H, generator=g) * 1.5            # large enough for the swigluoai clamps to bite
+    w13 = torch.randn(E, 2 * I, H, generator=g) * 0.4
+    w2 = torch.randn(E, H, I, generator=g) * 0.2
+    b13 = torch.randn(E, 2 * I, generator=g) if bias else None
+    b2 = torch.randn(E, H, generator=g) if bias else None
+    ids = torch.randint(0, E, (T, 1), generator=g).int()
+    w = torch.rand(T, 1, generator=g) + 0.25
+    out = oracle.fused_experts_ref(x, w13, w2, w, ids, activation=act, w1_bias=b13, w2_bias=b2,
+                                   apply_router_weight_on_input=on_input)
+    want = torch.zeros(T, H, dtype=torch.float64)
+    for e in range(E):
+        sel = (ids[:, 0] == e).nonzero().flatten()
+        want[sel] = _mlp64(x[sel], w13[e], w2[e], act, None if b13 is None else b13[e],
+                           None if b2 is None else b2[e],
+                           in_weight=w[sel, 0] if on_input else None,
+                           out_weight=None if on_input else w[sel, 0])
+    if act == "swigluoai":
+        assert (x @ w13[0].t()).abs().max() > 7.0       # the clamp is exercised
+    assert torch.allclose(out.double(), want, rtol=2e-5, atol=2e-5)
+    # the two sides of the weight differ (the activation is not linear), so the flag matters
+    other = oracle.fused_experts_ref(x, w13, w2, w, ids, activation=act, w1_bias=b13, w2_bias=b2,
+                                     apply_router_weight_on_input=not on_input)
+    assert not torch.allclose(out, other, rtol=1e-3, atol=1e-3)
+
+
+def test_fused_experts_topk_combine_is_the_plain_sum(oracle):
+    """K=3: the result is the sum over k of the K=1 results (moe_easy_kernel.py:26-31),
+    and a bias on the down projection is counted once per selected expert, scaled by
+    that expert's routed weight."""
+    E, H, I, T, K = 5, 32, 24, 17, 3
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(T, H, generator=g)
+    w13 = torch.randn(E, 2 * I, H, generator=g) * 0.3
+    w2 = torch.randn(E, H, I, generator=g) * 0.3
+    b2 = torch.randn(E, H, generator=g)
+    logits = torch.randn(T, E, generator=g)
+    w, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
+    out = oracle.fused_experts_ref(x, w13, w2, w, ids, w2_bias=b2)
+    parts = sum(oracle.fused_experts_ref(x, w13, w2, w[:, k:k + 1], ids[:, k:k + 1], w2_bias=b2)
+                for k in range(K))
+    assert torch.allclose(out, parts, rtol=1e-5, atol=1e-6)
+    want = torch.zeros(T, H, dtype=torch.float64)
+    for t in range(T):
+        for k in range(K):
+            e = ids[t, k].item()
+            want[t] += _mlp64(x[t:t + 1], w13[e], w2[e], "silu", b2=b2[e], out_weight=w[t:t + 1, k])[0]
+    assert torch.allclose(out.double(), want, rtol=2e-5, atol=2e-5)
+
+
+def _bf(v):
+    return torch.as_tensor(v, dtype=torch.float32).bfloat16().float()
+
+
+def test_mirror_rounding_step_by_step_on_a_2x2_case(oracle):
+    """Every rounding point of the two mirrored modes on a case small enough to
+    follow by hand (H = 2, I = 1, E = 1, K = 1): the values are chosen so that each
+    rounding changes the bf16 result, hence a missing or extra rounding fails."""
+    x = torch.tensor([[1.5390625, -0.29296875]]).bfloat16()
+    w13 = torch.tensor([[[-2.171875, 0.5703125], [-1.0859375, -1.3984375]]]).bfloat16()   # gate row, up row
+    w2 = torch.tensor([[[0.404296875], [0.83984375]]]).bfloat16()
+    tw = torch.tensor([[0.7]])
+    ids = torch.zeros(1, 1, dtype=torch.int32)
+    xf, w13f, w2f = x.float(), w13.float(), w2.float()
+    gate32 = xf[0, 0] * w13f[0, 0, 0] + xf[0, 1] * w13f[0, 0, 1]
+    up32 = xf[0, 0] * w13f[0, 1, 0] + xf[0, 1] * w13f[0, 1, 1]
+    silu = lambda v: v / (1 + torch.exp(-v))
+    # mirror_rounding=True: GEMM1 -> bf16, silu -> bf16, product -> bf16, weighted GEMM2 -> bf16, sum -> bf16
+    g16, u16 = _bf(gate32), _bf(up32)
+    assert g16 != gate32 and u16 != up32                              # the first rounding bites
+    s16 = _bf(oracle.silu_and_mul(torch.stack([g16, torch.tensor(1.0)])[None].bfloat16()).float()[0, 0])
+    assert s16 == _bf(silu(g16)) and s16 != silu(g16)
+    c2 = _bf(s16 * u16)
+    assert c2 != s16 * u16
+    want_true = torch.stack([_bf(_bf((c2 * w2f[0, r, 0]) * tw[0, 0])) for r in range(2)])
+    got_true = oracle.fused_experts_ref(x, w13, w2, tw, ids, mirror_rounding=True)
+    assert torch.equal(got_true[0], want_true)
+    # mirror_rounding="fused": silu(gate) * up on the fp32 sums, one rounding
+    c2f = _bf(silu(gate32) * up32)
+    want_fused = torch.stack([_bf((c2f * w2f[0, r, 0]) * tw[0, 0]) for r in range(2)])
+    got_fused = oracle.fused_experts_ref(x, w13, w2, tw, ids, mirror_rounding="fused")
+    assert torch.equal(got_fused[0], want_fused)
+    assert c2f != c2 and not torch.equal(got_fused, got_true)         # the modes are told apart here
+    # and the pure fp32 mode rounds nowhere
+    want32 = torch.stack([(silu(gate32) * up32 * w2f[0, r, 0]) * tw[0, 0] for r in range(2)])
+    got32 = oracle.fused_experts_ref(x, w13, w2, tw, ids)
+    assert torch.allclose(got32[0], want32, rtol=1e-6, atol=0) and not torch.equal(got32, got_fused)
+
+
+# ----------------------------------------------------------------- fp8 expert MLP
+def _fp8_cast(t):
+    """torch's own e4m3fn rounding (saturating inputs are never passed)."""
+    return t.to(torch.float8_e4m3fn).float()
+
+
+def _fp8_layer(seed, E=3, H=64, I=32, T=21):
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(T, H, generator=g) * torch.logspace(-2, 2, T)[:, None]).bfloat16()   # rows of very different size
+    # output channels of very different size: a scale applied along the wrong axis cannot pass
+    w13 = torch.randn(E, 2 * I, H, generator=g) * 0.2 * (2.0 ** (torch.arange(2 * I) % 7 - 3))[None, :, None]
+    w2 = torch.randn(E, H, I, generator=g) * 0.2 * (2.0 ** (torch.arange(H) % 5 - 2))[None, :, None]
+    return x, w13, w2, g
+
+
+def test_fp8_reference_step_by_step_against_library_routines(oracle):
+    """K=1: per token, x is quantised per row, multiplied with the dequantised
+    per-channel weights, gated, quantised per row *again* and multiplied with the
+    dequantised down weights.  Every step here uses torch's e4m3 cast and
+    F.linear, with wildly non-uniform row and channel magnitudes, so a scale on
+    the wrong axis, a missing second quantisation, a dropped routed weight or a
+    static (per-tensor) activation scale each fail."""
+    F = torch.nn.functional
+    x, w13, w2, g = _fp8_layer(5)
+    E, T, I = w13.shape[0], x.shape[0], w2.shape[2]
+    q13, s13 = oracle.quant_weight_per_channel(w13)
+    q2, s2 = oracle.quant_weight_per_channel(w2)
+    assert s13.shape == (E, 2 * I) and s2.shape == (E, w2.shape[1])
+    assert s13.max() / s13.min() > 30 and s2.max() / s2.min() > 8
+    ids = torch.randint(0, E, (T, 1), generator=g).int()
+    tw = torch.rand(T, 1, generator=g) + 0.25
+    got = oracle.fused_experts_fp8_ref(x, q13, s13, q2, s2, tw, ids)
+    xf = x.float()
+    sx = xf.abs().amax(-1) / 448.0
+    xd = _fp8_cast(xf * (1.0 / sx)[:, None]) * sx[:, None]
+    want = torch.zeros(T, w2.shape[1])
+    for t in range(T):
+        e = ids[t, 0].item()
+        W1 = _fp8_cast(w13[e] * (1.0 / s13[e])[:, None]) * s13[e][:, None]
+        W2 = _fp8_cast(w2[e] * (1.0 / s2[e])[:, None]) * s2[e][:, None]
+        h = F.linear(xd[t], W1)
+        a = F.silu(h[:I]) * h[I:]
+        sa = a.abs().amax() / 448.0
+        ad = _fp8_cast(a * (1.0 / sa)) * sa
+        want[t] = F.linear(ad, W2) * tw[t, 0]
+    assert torch.allclose(got, want, rtol=1e-4, atol=1e-6 * want.abs().max().item())
+    # without the second quantisation the result is measurably different
+    nore = torch.zeros_like(want)
+    for t in range(T):
+        e = ids[t, 0].item()
+        W1 = oracle.dequant_e4m3(q13[e]) * s13[e][:, None]
+        W2 = oracle.dequant_e4m3(q2[e]) * s2[e][:, None]
+        h = F.linear(xd[t], W1)
+        nore[t] = F.linear(F.silu(h[:I]) * h[I:], W2) * tw[t, 0]
+    assert not torch.allclose(got, nore, rtol=1e-3, atol=1e-3 * want.abs().max().item())
+
+
+def test_fp8_reference_equals_the_16bit_reference_up_to_one_requantisation(oracle):
+    """Weights and activations that e4m3 holds exactly (code values times a
+    power-of-two row scale) pass through both quantisers unchanged, so the fp8
+    reference may differ from ``fused_experts_ref`` on the same tensors only by
+    the re-quantisation of the gated intermediate: at most half an e4m3 step
+    (2^-4 relative; 2^-10 of the row scale in the subnormal range) per element,
+    propagated through |W2|."""
+    g = torch.Generator().manual_seed(8)
+    E, H, I, T, K = 4, 64, 32, 26, 2
+    codes = torch.tensor([c for c in range(256) if (c & 0x7f) not in (0x7f,)], dtype=torch.uint8)
+    vals = oracle.dequant_e4m3(codes)
+
+    def exact(shape, row_exp):
+        pick = vals[torch.randint(0, vals.numel(), shape, generator=g)]
+        pick[..., 0] = 448.0                               # every row reaches the largest code
+        return pick * (2.0 ** row_exp)[..., None]
+
+    x = exact((T, H), torch.randint(-12, -6, (T,), generator=g).float()).bfloat16()
+    w13 = exact((E, 2 * I, H), torch.randint(-14, -9, (E, 2 * I), generator=g).float())
+    w2 = exact((E, H, I), torch.randint(-13, -8, (E, H), generator=g).float())
+    assert torch.equal(x.float().bfloat16(), x)            # 4-bit mantissas: bf16 holds them
+    q13, s13 = oracle.quant_weight_per_channel(w13)
+    q2, s2 = oracle.quant_weight_per_channel(w2)
+    assert torch.equal(oracle.dequant_e4m3(q13) * s13[..., None], w13)      # lossless
+    assert torch.equal(oracle.dequant_e4m3(q2) * s2[..., None], w2)
+    xq, xs = oracle.quant_act_per_token(x)
+    assert torch.equal(oracle.dequant_e4m3(xq) * xs[:, None], x.float())
+    logits = torch.randn(T, E, generator=g)
+    tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
+    got = oracle.fused_experts_fp8_ref(x, q13, s13, q2, s2, tw, ids)
+    ref = oracle.fused_experts_ref(x.float(), w13, w2, tw, ids)
+    bound = torch.zeros(T, H)
+    for t in range(T):
+        for k in range(K):
+            e = ids[t, k].item()
+            h = w13[e] @ x[t].float()
+            a = torch.nn.functional.silu(h[:I]) * h[I:]
+            step = torch.maximum(a.abs() * 2.0 ** -4, (a.abs().amax() / 448.0) * 2.0 ** -10)
+            bound[t] += tw[t, k] * (w2[e].abs() @ step)
+    err = (got - ref).abs()
+    assert (err <= bound * 1.001 + 1e-7 * ref.abs().max()).all()
+    assert err.max() > 0.05 * bound.max()                  # and the re-quantisation is really there
+
+
+def test_fp8_mirrored_modes_round_where_the_kernels_store(oracle):
+    """mirror_rounding=True / "fused" of the fp8 reference: same steps as the
+    library recomputation above with the 16-bit roundings inserted."""
+    F = torch.nn.functional
+    x, w13, w2, g = _fp8_layer(9, E=2, T=9)
+    I = w2.shape[2]
+    q13, s13 = oracle.quant_weight_per_channel(w13)
+    q2, s2 = oracle.quant_weight_per_channel(w2)
+    ids = torch.randint(0, 2, (9, 1), generator=g).int()
+    tw = torch.rand(9, 1, generator=g) + 0.25
+    xf = x.float()
+    sx = xf.abs().amax(-1) / 448.0
+    xd = _fp8_cast(xf * (1.0 / sx)[:, None]) * sx[:, None]
+    r16 = lambda t: t.bfloat16().float()
+    for mode in (True, "fused"):
+        got = oracle.fused_experts_fp8_ref(x, q13, s13, q2, s2, tw, ids, mirror_rounding=mode)
+        want = torch.zeros_like(got)
+        for t in range(9):
+            e = ids[t, 0].item()
+            W1 = oracle.dequant_e4m3(q13[e]) * s13[e][:, None]
+            W2 = oracle.dequant_e4m3(q2[e]) * s2[e][:, None]
+            h = F.linear(xd[t], W1)
+            if mode is True:
+                h = r16(h)
+                a = r16(r16(oracle.silu_and_mul(torch.cat([h[:I], torch.ones(I)])[None].bfloat16()).float()[0])
+                        * h[I:])
+            else:
+                a = r16(h[:I] / (1 + torch.exp(-h[:I])) * h[I:])
+            sa = a.abs().amax() / 448.0
+            ad = _fp8_cast(a * (1.0 / sa)) * sa
+            want[t] = r16(r16(F.linear(ad, W2) * tw[t, 0]))
+        assert torch.allclose(got, want, rtol=2.0 ** -7, atol=1e-6 * want.abs().max().item()), mode
+        assert (got != want).float().mean() < 0.02, mode    # only fp32 summation order can flip a rounding
+
+
+def test_quantiser_scale_floor_for_near_subnormal_rows(oracle):
+    """A row whose largest magnitude is tiny but not zero: amax / 448 would have a
+    reciprocal that overflows (zeros would turn into NaN codes, the rest saturate).
+    The scale is floored at 2^-100 instead; codes stay finite and the round trip is
+    still within half an e4m3 step of that scale."""
+    x = torch.zeros(4, 16)
+    x[0, 3] = 1e-38                     # 1 / (amax / 448) would be +inf
+    x[0, 4] = 1e-40                     # subnormal input
+    x[1, 5] = -192 * 2.0 ** -100
+    x[1, 6] = 2.0 ** -109               # smallest e4m3 subnormal at the floor scale
+    x[2, 1] = 448 * 2.0 ** -100         # exactly at the floor
+    q, s = oracle.quant_act_per_token(x)
+    assert s.tolist() == [2.0 ** -100, 2.0 ** -100, 2.0 ** -100, 1.0]
+    assert not ((q & 0x7f) == 0x7f).any()                     # no NaN code
+    assert q[3].count_nonzero() == 0 and q[0].count_nonzero() == 0 and q[2, 1] == 0x7e
+    assert q[1, 5] == (0x80 | 0x74) and q[1, 6] == 0x01       # -192 = -1.5 * 2^7; 2^-9
+    d = oracle.dequant_e4m3(q) * s[:, None]
+    assert ((d - x).abs() <= 2.0 ** -100 * 2.0 ** -10 + x.abs() * 2.0 ** -4).all()
+    qw, sw = oracle.quant_weight_per_channel(x[None])
+    assert torch.equal(qw[0], q) and torch.equal(sw[0], s)
