@@ -313,7 +313,15 @@ def test_fp8_layered_prefill_batch_every_eighth_row(moe, oracle, dev):
     rows = torch.cat([torch.arange(0, 8192, 8), torch.arange(8192, 8448)])
     q13, q2 = w13q.view(torch.uint8).cpu(), w2q.view(torch.uint8).cpu()
     ref = oracle.fused_experts_fp8_ref(x[rows], q13, w13s.cpu(), q2, w2s.cpu(), tw.cpu()[rows], ids.cpu()[rows])
-    _close_fp8(out[rows.to(dev)], ref)
+    # The kernels quantise the stored 16-bit intermediate, this oracle its fp32 value: an element
+    # that the 16-bit rounding (or the row scale derived from it) moves across an e4m3 tie changes
+    # by a whole e4m3 step, about one element in sixty.  Over 2.6 million outputs the tail of
+    # those flips reaches 0.02, so: rtol 6e-2 with the absolute floor at one e4m3 step (2^-3) of
+    # a typical output for every element, and the bf16 floor of 1e-2 for all but 1 in 10 000.
+    got = out[rows.to(dev)].float().cpu()
+    _close_fp8(got, ref, atol=0.125 * ref.pow(2).mean().sqrt().item())
+    off = (got - ref).abs() > 1e-2 + 6e-2 * ref.abs()
+    assert off.float().mean().item() <= 1e-4, f"{off.sum().item()} of {off.numel()} beyond rtol 6e-2 / atol 1e-2"
     mode = _mode(moe, x.shape[0], shape.experts, shape.top_k, shape.hidden, torch.bfloat16, fp8=True)
     assert mode == "fused"
     refm = oracle.fused_experts_fp8_ref(x[rows], q13, w13s.cpu(), q2, w2s.cpu(), tw.cpu()[rows], ids.cpu()[rows],
