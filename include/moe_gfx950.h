@@ -89,6 +89,22 @@ int moe_align_block_size(const void* topk_ids, int ids_dtype, int64_t numel, int
                          int32_t* expert_ids, int64_t expert_cap, int32_t* num_tokens_post_pad,
                          void* workspace, int64_t workspace_bytes, void* stream);
 
+/* moe_align_block_size without a workspace argument and without any allocation.  No
+ * counterpart in the reference; it is for callers that cannot allocate: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  The scratch the
+ * large path needs (per-segment histograms, moe_align_workspace_bytes) lives in a 4 MiB
+ * device array inside the library, one copy per GPU, held until the process ends; sizes
+ * that need more are rejected with MOE_ERR_WORKSPACE (at 128 experts the limit is about
+ * 4 million ids, at 1024 experts about 520 thousand).  Every call on a GPU shares that
+ * GPU's array: calls that overlap on one GPU (two streams, two threads) race; calls on one
+ * stream are ordered and each call overwrites what it reads, so nothing needs clearing.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress); make that
+ * call outside graph capture.  Results are those of moe_align_block_size, bit for bit. */
+int moe_align_block_size_static(const void* topk_ids, int ids_dtype, int64_t numel, int E,
+                                int block_size, int32_t* sorted_token_ids, int64_t sorted_cap,
+                                int32_t* expert_ids, int64_t expert_cap,
+                                int32_t* num_tokens_post_pad, void* stream);
+
 /* The same alignment for block_size 256, which also leaves in the workspace of the
  * moe_fused_experts call that follows what that call would otherwise compute with a launch
  * of its own: the per-XCD m-block ranges of the large-tile kernel (`plan_bounds`, 9 int32)

@@ -28,7 +28,7 @@ EXPORTS = (
     "moe_fused_experts_workspace_bytes", "moe_fused_experts", "moe_preferred_block_size",
     "moe_quant_rows_e4m3", "moe_gate_topk_softmax", "moe_add_rms_norm",
     "moe_align_can_plan", "moe_align_block_size_planned", "moe_fused_experts_plan_layout",
-    "moe_fused_experts_status", "moe_fused_experts_set_wait_limit",
+    "moe_fused_experts_status", "moe_fused_experts_set_wait_limit", "moe_align_block_size_static",
 )
 
 
@@ -76,6 +76,8 @@ def _declare(L: ctypes.CDLL) -> None:
     L.moe_align_workspace_bytes.argtypes = [i64, i32]
     L.moe_align_block_size.restype = i32
     L.moe_align_block_size.argtypes = [p, i32, i64, i32, i32, p, i64, p, i64, p, p, i64, p]
+    L.moe_align_block_size_static.restype = i32
+    L.moe_align_block_size_static.argtypes = [p, i32, i64, i32, i32, p, i64, p, i64, p, p]
     L.moe_align_can_plan.restype = i32
     L.moe_align_can_plan.argtypes = [i64, i32]
     L.moe_align_block_size_planned.restype = i32

@@ -552,3 +552,51 @@ MOE_EXPORT int moe_align_block_size_planned(const void* topk_ids, int ids_dtype,
                     expert_cap, num_tokens_post_pad, workspace, workspace_bytes, stream, plan_bounds,
                     plan_done, plan_num_done, plan_cap_mb);
 }
+
+// ---------------------------------------------------------------------------
+// Allocation-free variant: the per-segment histograms of the large path live in a
+// file-scope device array instead of a caller-provided workspace.  Each GPU the
+// library runs on holds its own copy of the array (at its own address) until the
+// process ends.
+// ---------------------------------------------------------------------------
+constexpr int64_t kStaticScratchBytes = 4 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+// device address of `scratch` per device; the array's name is only a host-side handle
+static std::atomic<void*> g_scratch_ptr[kMoeMaxDevices];
+
+static int static_scratch(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return moe_fail(MOE_ERR_LAUNCH, "moe_align_block_size_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMoeMaxDevices)
+    return moe_fail(MOE_ERR_UNSUPPORTED, "moe_align_block_size_static: device %d beyond the %d this entry point tracks", dev, kMoeMaxDevices);
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    // once per device, with that device current
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return moe_fail(MOE_ERR_LAUNCH, "moe_align_block_size_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // two threads storing the same address is harmless
+  }
+  *out = p;
+  return MOE_OK;
+}
+
+MOE_EXPORT int moe_align_block_size_static(const void* topk_ids, int ids_dtype, int64_t numel, int E,
+                                           int block_size, int32_t* sorted_token_ids, int64_t sorted_cap,
+                                           int32_t* expert_ids, int64_t expert_cap,
+                                           int32_t* num_tokens_post_pad, void* stream) {
+  const int64_t need = moe_align_workspace_bytes(numel, E);
+  if (need > kStaticScratchBytes)
+    return moe_fail(MOE_ERR_WORKSPACE, "moe_align_block_size_static: %lld ids over %d experts need %lld B of scratch, "
+                    "the built-in buffer holds %lld B; use moe_align_block_size with a workspace",
+                    static_cast<long long>(numel), E, static_cast<long long>(need),
+                    static_cast<long long>(kStaticScratchBytes));
+  void* ws = nullptr;
+  if (need > 0) {
+    if (int rc = static_scratch(&ws)) return rc;
+  }
+  // the count kernel writes every histogram entry the later kernels read: nothing has to start at zero
+  return align_impl(topk_ids, ids_dtype, numel, E, block_size, sorted_token_ids, sorted_cap, expert_ids,
+                    expert_cap, num_tokens_post_pad, ws, need, stream, nullptr, nullptr, 0, 0);
+}

@@ -110,6 +110,29 @@ def moe_align_block_size(topk_ids: torch.Tensor, num_experts: int, block_size: i
                              num_tokens_post_pad, None)
 
 
+def moe_align_block_size_static(topk_ids: torch.Tensor, num_experts: int, block_size: int,
+                                sorted_token_ids: torch.Tensor, experts_ids: torch.Tensor,
+                                num_tokens_post_pad: torch.Tensor) -> None:
+    """``moe_align_block_size`` through the entry point that allocates nothing
+    (``moe_align_block_size_static``): its scratch is a fixed device array inside the
+    library, so neither the library nor this wrapper allocates.  For callers that cannot
+    allocate; no counterpart in the reference.  Sizes beyond the built-in scratch raise."""
+    require_gpu_tensor(topk_ids, "topk_ids")
+    if topk_ids.dtype not in _lib.ID_DTYPE_CODE:
+        raise RuntimeError(f"moe_align_block_size_kernel not implemented for '{topk_ids.dtype}'")
+    for name, t in (("sorted_token_ids", sorted_token_ids), ("experts_ids", experts_ids),
+                    ("num_tokens_post_pad", num_tokens_post_pad)):
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be a contiguous int32 tensor")
+    if not topk_ids.is_contiguous():
+        raise RuntimeError("topk_ids must be contiguous")
+    with torch.cuda.device(topk_ids.device):
+        check(lib().moe_align_block_size_static(
+            topk_ids.data_ptr(), _lib.ID_DTYPE_CODE[topk_ids.dtype], topk_ids.numel(), num_experts,
+            block_size, sorted_token_ids.data_ptr(), sorted_token_ids.numel(), experts_ids.data_ptr(),
+            experts_ids.numel(), num_tokens_post_pad.data_ptr(), stream_ptr(topk_ids.device)))
+
+
 def align_block_size_planned(topk_ids: torch.Tensor, num_experts: int, block_size: int,
                              sorted_token_ids: torch.Tensor, experts_ids: torch.Tensor,
                              num_tokens_post_pad: torch.Tensor, plan) -> None:
