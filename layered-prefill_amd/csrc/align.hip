@@ -146,7 +146,7 @@ __device__ __forceinline__ void scatter_segment(const void* ids, int dtype, int6
 // What big_plan_kernel (grouped_gemm.hip) derives from the aligned ids, derived from the
 // per-expert counts instead, for an alignment with blocks of 256 slots: the m-block
 // ranges [bounds[x], bounds[x+1]) of the 8 XCDs with equal estimated work (a block costs
-// 36 / 45 / 62 / 64 with at most 32 / at most 64 / fewer than 256 / 256 real slots), no range
+// 38 / 48 / 64 / 64 with at most 32 / at most 64 / fewer than 256 / 256 real slots), no range
 // longer than cap_mb, and the per-block counters and the status word of the one-launch form
 // cleared.  Saves the
 // large-tile path a launch.  Called by all kScanThreads threads; contains barriers.
@@ -163,7 +163,7 @@ __device__ void plan_from_counts(const volatile int* cum, const volatile int* to
     first = cum[threadIdx.x] / kPlanBlock;
     if (nb > 0) {
       const int r = tot[threadIdx.x] - (nb - 1) * kPlanBlock;  // real slots of the expert's last block
-      w = (nb - 1) * 64 + (r <= 32 ? 36 : (r <= 64 ? 45 : (r < kPlanBlock ? 62 : 64)));
+      w = (nb - 1) * 64 + (r <= 32 ? 38 : (r <= 64 ? 48 : 64));
     }
   }
   const int excl = block_exclusive_scan(w, wave_tot);

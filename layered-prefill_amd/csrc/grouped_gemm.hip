@@ -21,7 +21,7 @@
 
 #ifdef MOE_TRACE
 // Development aid (make EXTRA=-DMOE_TRACE): per-workgroup phase timestamps of the large-tile kernel.
-__device__ unsigned long long moe_dbg[8 * 4096 + 4 * 128 + 4 * 4096];
+__device__ unsigned long long moe_dbg[12 * 16384];
 #define MOE_TRACE_NOW() __builtin_amdgcn_s_memrealtime()
 #else
 #define MOE_TRACE_NOW() 0ull
@@ -137,7 +137,15 @@ struct GemmParams {
   int m_major;       // workgroup order inside an XCD: all n-tiles of an m-block are neighbours
   const int32_t* xcd_bounds;  // large-tile kernel: m-block range [b[x], b[x+1]) of XCD x, or null
   int wt_stores;     // large-tile flush: results go out as device-scope write-through stores (one-launch hand-off)
+#ifdef MOE_DEV
+  int dev;           // development switches (MOE_DEV_FLAGS), never in a shipped build
+#endif
 };
+#ifdef MOE_DEV
+#define MOE_DEV_BIT(p, b) (((p).dev >> (b)) & 1)
+#else
+#define MOE_DEV_BIT(p, b) 0
+#endif
 
 constexpr int kThreads = 256;
 constexpr int kBK = 64;                  // K elements per LDS tile
@@ -491,12 +499,33 @@ struct BigCtx {
 template <int V>
 struct IntTag { static constexpr int value = V; };
 
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (B < E) {
+    f(IntTag<B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+
+// 16 bytes per lane from global memory into LDS at unit_lds + GROUP * 4096 + 16 * lane: the
+// destination offset goes into M0 with one scalar addition, the wait state M0 needs is the s_nop.
+template <int GROUP>
+__device__ __forceinline__ void lds_dma16_group(const char* base, uint32_t lane_byte_offset, uint32_t unit_lds) {
+  asm volatile(
+      "s_add_u32 m0, %0, %3\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, %2"
+      :
+      : "s"(unit_lds), "v"(lane_byte_offset), "s"(base), "n"(GROUP * 4096)
+      : "memory", "scc");
+}
+
 // Main loop for a wavefront that has FMC live token fragments (0..4).
 // Unit j of the stream  A(0) W(0) A(1) W(1) ...  lives in ring slot j % 5.
-// The caller has requested W(0) and W(1) (when nk > 1) before anything else.
-// One K tile (128 bytes per row) is STEPS MFMA steps of CH 16-byte chunks per
-// lane and operand: four steps of one chunk for the 16-bit dtypes, two steps
-// of two chunks for e4m3.  Two register sets of fragments (P, Q) alternate,
+// The caller has requested W(0) and the first half of W(1) (when nk > 1) before
+// anything else.  One K tile (128 bytes per row) is STEPS MFMA steps of CH 16-byte
+// chunks per lane and operand: four steps of one chunk for the 16-bit dtypes, two
+// steps of two chunks for e4m3.  Two register sets of fragments (P, Q) alternate,
 // and every step carries, between its MFMAs, the LDS reads of the next step's
 // fragments and its share of the sixteen DMA requests of the K tile:
 //   steps 0 .. STEPS-2 of tile kt request W(kt+1)[4..7] and A(kt+2)[0..7]
@@ -504,148 +533,169 @@ struct IntTag { static constexpr int value = V; };
 //   step STEPS-1 reads P(kt+1,0) and requests W(kt+2)[0..3]
 // At the wait only A(kt+2), the youngest request, may still be outstanding.
 // sched_barrier pins this order against the compiler's scheduler.
-template <typename Mma, int FMC>
+// The loop is bound by instruction issue (one wavefront per SIMD issues one
+// instruction every four clocks, an MFMA takes 32), so a K tile is straight-line
+// code: the two tiles at the end of K, which request less, are separate
+// instances of the tile body instead of tests around every request, an LDS read
+// is one instruction (lane base + slot in one addition per operand and step,
+// everything else in the offset field), a DMA request three.
+template <typename Mma, int FMC, bool GATED>
 __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, int nk,
                                              f32x16 (&acc)[4][4]) {
   constexpr int CH = Mma::kBigChunks, STEPS = 4 / CH;
   constexpr int PER = 12 / (STEPS - 1);  // requests carried by each of the first STEPS-1 steps
-  auto dma_a = [&](int kt, int slot, int i) {
-    lds_dma16(c.a_base + kt * kBigRowBytes, c.a_off[i], c.dma_lds + slot * kBigUnitBytes + i * 4096);
-  };
-  auto dma_w = [&](int kt, int slot, int i) {
-    lds_dma16(c.w_base + kt * kBigRowBytes, c.w_off[i], c.dma_lds + slot * kBigUnitBytes + i * 4096);
-  };
-  auto issue_a = [&](int kt, int slot) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) dma_a(kt, slot, i);
-  };
   constexpr int XF = FMC > 0 ? FMC : 1;
-  auto read_frags = [&](int sa, int sw, int kk, uint4 (&wf)[4][CH], uint4 (&xf)[XF][CH]) {
-    if constexpr (FMC > 0) {
+  constexpr int NM = 4 * FMC;            // MFMAs of a step
+  // byte offset of weight fragment fn from fragment 0 inside a weight unit
+  auto woff = [](int fn) { return GATED ? (fn < 2 ? fn * 4096 : 16384 + (fn - 2) * 4096) : fn * 4096; };
+  // per-lane parts of the fragment addresses: chunk q of the K tile, token rows / weight rows
+  int xl[4], wl[4];
 #pragma unroll
-      for (int ch = 0; ch < CH; ++ch) {
-        const char* stw = smem + sw * kBigUnitBytes + c.rd_k[kk * CH + ch];
-        const char* sta = smem + sa * kBigUnitBytes + c.x_row + c.rd_k[kk * CH + ch];
-#pragma unroll
-        for (int fn = 0; fn < 4; ++fn) wf[fn][ch] = *reinterpret_cast<const uint4*>(stw + c.w_row[fn]);
-#pragma unroll
-        for (int fm = 0; fm < FMC; ++fm)
-          xf[fm][ch] = *reinterpret_cast<const uint4*>(sta + fm * 32 * kBigRowBytes);
-      }
-    }
-  };
-  // One MFMA step on fragment set X.  The LDS reads of the next step's set Y
-  // and ND DMA requests are spread between its MFMAs instead of being issued
-  // back to back: the LDS and the vector memory path each take one wavefront
-  // request every few dozen clocks when all four wavefronts stream, so a burst
-  // stalls the wavefront, and with it the matrix pipe, until the queue drains.
-  // Reads go out in the order the next step consumes them.
-  auto step = [&](auto nd_tag, const uint4 (&wfX)[4][CH], const uint4 (&xfX)[XF][CH], uint4 (&wfY)[4][CH],
-                  uint4 (&xfY)[XF][CH], bool load_y, int ya, int yw, int ykk, auto&& dma) {
+  for (int q = 0; q < 4; ++q) {
+    xl[q] = c.x_row + c.rd_k[q];
+    wl[q] = c.w_row[0] + c.rd_k[q];
+  }
+  uint4 wfP[4][CH], xfP[XF][CH], wfQ[4][CH], xfQ[XF][CH];
+#ifdef MOE_TRACE
+  unsigned long long tr_v = 0, tr_b = 0;
+  const unsigned long long tr0 = __builtin_readcyclecounter();
+#endif
+
+  // One MFMA step on fragment set X.  Between its MFMAs: the LDS reads of set Y (chunks of
+  // MFMA step YKK of the tile whose units start at byte ya / yw of the ring) when LOAD, and
+  // requests [0, ND) of `dma`.  Spread out, because a burst of requests stalls the wavefront,
+  // and with it the matrix pipe, until the queue drains.  Reads go out in the order the next
+  // step consumes them: x0, w0..w3, x1, x2, x3.
+  auto step = [&](auto nd_tag, auto load_tag, auto ykk_tag, const uint4 (&wfX)[4][CH], const uint4 (&xfX)[XF][CH],
+                  uint4 (&wfY)[4][CH], uint4 (&xfY)[XF][CH], int ya, int yw, auto&& dma) {
     constexpr int ND = decltype(nd_tag)::value;
-    auto read_y = [&](int r) {  // r: 0 x0, 1..4 w0..w3, 5.. x1..
-      if constexpr (FMC > 0) {
-        if (!load_y) return;
+    constexpr bool LOAD = decltype(load_tag)::value != 0 && FMC > 0;
+    constexpr int YKK = decltype(ykk_tag)::value;
+    auto read_y = [&](auto rt) {
+      constexpr int r = decltype(rt)::value;
+      if constexpr (LOAD) {
 #pragma unroll
         for (int ch = 0; ch < CH; ++ch) {
-          const char* stw = smem + yw * kBigUnitBytes + c.rd_k[ykk * CH + ch];
-          const char* sta = smem + ya * kBigUnitBytes + c.x_row + c.rd_k[ykk * CH + ch];
-          if (r == 0) xfY[0][ch] = *reinterpret_cast<const uint4*>(sta);
-          else if (r <= 4) wfY[r - 1][ch] = *reinterpret_cast<const uint4*>(stw + c.w_row[r - 1]);
-          else if (r - 4 < FMC) xfY[r - 4][ch] = *reinterpret_cast<const uint4*>(sta + (r - 4) * 32 * kBigRowBytes);
+          const char* sta = smem + (ya + xl[YKK * CH + ch]);
+          const char* stw = smem + (yw + wl[YKK * CH + ch]);
+          if constexpr (r == 0) xfY[0][ch] = *reinterpret_cast<const uint4*>(sta);
+          else if constexpr (r <= 4) wfY[r - 1][ch] = *reinterpret_cast<const uint4*>(stw + woff(r - 1));
+          else if constexpr (r - 4 < FMC) xfY[r - 4][ch] = *reinterpret_cast<const uint4*>(sta + (r - 4) * 4096);
         }
       }
     };
-    constexpr int NM = 4 * FMC;  // MFMAs of this step
-#pragma unroll
-    for (int m = 0; m < (NM > 0 ? NM : 1); ++m) {
-      if constexpr (NM > 0) {
-        const int fm = m >> 2, fn = m & 3;
-        acc[fn][fm] = Mma::mma_big(wfX[fn], xfX[fm], acc[fn][fm]);
-      }
+    static_for<0, (NM > 0 ? NM : 1)>([&](auto mt) {
+      constexpr int m = decltype(mt)::value;
+      if constexpr (NM > 0) acc[m & 3][m >> 2] = Mma::mma_big(wfX[m & 3], xfX[m >> 2], acc[m & 3][m >> 2]);
       __builtin_amdgcn_sched_barrier(0);
-      if ((m & 1) == 0) read_y(m >> 1);
-#pragma unroll
-      for (int j = (m * ND) / 16; j < ((m + 1) * ND) / 16; ++j) dma(j);
+      if constexpr ((m & 1) == 0) read_y(IntTag<(m >> 1)>{});
+      static_for<(m * ND) / 16, ((m + 1) * ND) / 16>([&](auto jt) { dma(jt); });
       __builtin_amdgcn_sched_barrier(0);
-    }
+    });
     // wavefronts with fewer live fragments have fewer MFMAs to hide requests behind
-#pragma unroll
-    for (int r = (NM + 1) / 2; r < 8; ++r) read_y(r);
-#pragma unroll
-    for (int j = ((NM > 0 ? NM : 1) * ND) / 16; j < ND; ++j) dma(j);
+    static_for<(NM + 1) / 2, 8>([&](auto rt) { read_y(rt); });
+    static_for<((NM > 0 ? NM : 1) * ND) / 16, ND>([&](auto jt) { dma(jt); });
     __builtin_amdgcn_sched_barrier(0);
   };
-  auto next_slot = [](int s) { return s + 2 >= kBigUnits ? s + 2 - kBigUnits : s + 2; };
-  using Tag4 = IntTag<4>;
-  using TagPer = IntTag<PER>;
 
-  // fill the ring: W(0) and W(1) were requested by the caller as soon as it knew the
-  // expert; A(0) A(1) A(2) follow here.  Then wait for tile 0 only.
-  issue_a(0, 0);
-  if (1 < nk) issue_a(1, 2);
-  if (2 < nk) issue_a(2, 4);
-  if (2 < nk) wait_vmcnt<2 * kBigDmaPerUnit>();
-  else if (1 < nk) wait_vmcnt<kBigDmaPerUnit>();
-  else wait_vmcnt<0>();
-  bare_barrier();
-  int sa = 0, sw = 1;  // slots of the tile being multiplied
-  int fa = 0, fw = 0;  // slots the previous tile left free: W(kt+1) goes to fa, A(kt+2) to fw
-  uint4 wfP[4][CH], xfP[XF][CH], wfQ[4][CH], xfQ[XF][CH];
-  read_frags(sa, sw, 0, wfP, xfP);
-  __builtin_amdgcn_sched_barrier(0);
-#ifdef MOE_TRACE
-  unsigned long long tr_v = 0, tr_b = 0, tr_i = 0;
-  const unsigned long long tr0 = __builtin_readcyclecounter();
-#endif
-  for (int kt = 0; kt < nk; ++kt) {
-    // requests of this K tile, in order: W(kt+1) second half, then A(kt+2); W(kt+1)'s
-    // first half went out behind the last MFMA step of tile kt-1
-    const bool do_w = kt >= 1 && kt + 1 < nk, do_a = kt >= 1 && kt + 2 < nk;
-    auto req = [&](int q) {
-      if (q < 4) { if (do_w) dma_w(kt + 1, fa, 4 + q); }
-      else { if (do_a) dma_a(kt + 2, fw, q - 4); }
+  // ring state, in bytes from the start of the ring: units of the tile being multiplied
+  // (sa, sw) and the two units the tile before it left free (fa, fw): W(kt+1) goes to fa,
+  // A(kt+2) to fw
+  auto next_slot = [](int s) { return s + 2 * kBigUnitBytes >= kBigUnits * kBigUnitBytes ? s + (2 - kBigUnits) * kBigUnitBytes : s + 2 * kBigUnitBytes; };
+  int sa = 0, sw = kBigUnitBytes, fa = 3 * kBigUnitBytes, fw = 4 * kBigUnitBytes;
+  const char* a2 = c.a_base + 2 * kBigRowBytes;  // rows of A(kt+2)
+  const char* w1 = c.w_base + kBigRowBytes;      // rows of W(kt+1)
+
+  // One K tile.  DO_W: W(kt+1)[4..7] is still to be requested; DO_A: A(kt+2) exists; NEXT:
+  // a tile follows; NEXT_W: W(kt+2) exists.
+  auto ktile = [&](auto do_w_tag, auto do_a_tag, auto next_tag, auto next_w_tag) {
+    constexpr bool DO_W = decltype(do_w_tag)::value != 0, DO_A = decltype(do_a_tag)::value != 0;
+    constexpr bool NEXT = decltype(next_tag)::value != 0, NEXT_W = decltype(next_w_tag)::value != 0;
+    const uint32_t lds_fa = c.dma_lds + fa, lds_fw = c.dma_lds + fw;
+    const char* const w2 = w1 + kBigRowBytes;
+    // request q of the tile's first STEPS-1 steps: W(kt+1)[4..7], then A(kt+2)[0..7]
+    auto req = [&](auto qt) {
+      constexpr int q = decltype(qt)::value;
+      if constexpr (q < 4) { if constexpr (DO_W) lds_dma16_group<4 + q>(w1, c.w_off[4 + q], lds_fa); }
+      else { if constexpr (DO_A) lds_dma16_group<q - 4>(a2, c.a_off[q - 4], lds_fw); }
     };
+    using One = IntTag<1>;
     if constexpr (STEPS == 4) {
-      step(TagPer{}, wfP, xfP, wfQ, xfQ, true, sa, sw, 1, [&](int j) { req(j); });
-      step(TagPer{}, wfQ, xfQ, wfP, xfP, true, sa, sw, 2, [&](int j) { req(PER + j); });
-      step(TagPer{}, wfP, xfP, wfQ, xfQ, true, sa, sw, 3, [&](int j) { req(2 * PER + j); });
+      step(IntTag<PER>{}, One{}, IntTag<1>{}, wfP, xfP, wfQ, xfQ, sa, sw, [&](auto jt) { req(jt); });
+      step(IntTag<PER>{}, One{}, IntTag<2>{}, wfQ, xfQ, wfP, xfP, sa, sw, [&](auto jt) { req(IntTag<PER + decltype(jt)::value>{}); });
+      step(IntTag<PER>{}, One{}, IntTag<3>{}, wfP, xfP, wfQ, xfQ, sa, sw, [&](auto jt) { req(IntTag<2 * PER + decltype(jt)::value>{}); });
     } else {
-      step(TagPer{}, wfP, xfP, wfQ, xfQ, true, sa, sw, 1, [&](int j) { req(j); });
+      step(IntTag<PER>{}, One{}, IntTag<1>{}, wfP, xfP, wfQ, xfQ, sa, sw, [&](auto jt) { req(jt); });
     }
-    bool next_w = false;
-    if (kt + 1 < nk) {
-      // tile kt+1 must have landed (only A(kt+2), the youngest request, may
-      // still be outstanding) and nobody reads the slots of tile kt any more
-      // (its last fragment reads have returned: lgkmcnt(0))
+    if constexpr (NEXT) {
+      // tile kt+1 must have landed (only A(kt+2), the youngest request, may still be
+      // outstanding) and nobody reads the slots of tile kt any more (its last fragment
+      // reads have returned: lgkmcnt(0))
 #ifdef MOE_TRACE
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       const unsigned long long tr1 = __builtin_readcyclecounter();
 #endif
-      if (kt + 2 < nk) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+      if constexpr (DO_A) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
       else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 #ifdef MOE_TRACE
       const unsigned long long tr2 = __builtin_readcyclecounter();
 #endif
       bare_barrier();
 #ifdef MOE_TRACE
-      const unsigned long long tr3 = __builtin_readcyclecounter();
-      tr_v += tr2 - tr1; tr_b += tr3 - tr2;
+      tr_v += tr2 - tr1; tr_b += __builtin_readcyclecounter() - tr2;
 #endif
       fa = sa;
       fw = sw;
       sa = next_slot(sa);
       sw = next_slot(sw);
-      next_w = kt + 2 < nk;
     }
     __builtin_amdgcn_sched_barrier(0);
-    step(Tag4{}, wfQ, xfQ, wfP, xfP, kt + 1 < nk, sa, sw, 0, [&](int i) { if (next_w) dma_w(kt + 2, fa, i); });
+    const uint32_t lds_w2 = c.dma_lds + fa;  // W(kt+2) takes the token unit of the tile just finished
+    step(IntTag<4>{}, IntTag<NEXT ? 1 : 0>{}, IntTag<0>{}, wfQ, xfQ, wfP, xfP, sa, sw, [&](auto it) {
+      constexpr int i = decltype(it)::value;
+      if constexpr (NEXT_W) lds_dma16_group<i>(w2, c.w_off[i], lds_w2);
+    });
+    a2 += kBigRowBytes;
+    w1 += kBigRowBytes;
+  };
+
+  // fill the ring: W(0) and half of W(1) were requested by the caller as soon as it knew
+  // the expert; A(0) and A(1) follow here.  Then wait for tile 0 only.
+  static_for<0, 8>([&](auto it) { lds_dma16_group<decltype(it)::value>(c.a_base, c.a_off[decltype(it)::value], c.dma_lds); });
+  if (1 < nk) {
+    static_for<0, 8>([&](auto it) {
+      lds_dma16_group<decltype(it)::value>(c.a_base + kBigRowBytes, c.a_off[decltype(it)::value], c.dma_lds + 2 * kBigUnitBytes);
+    });
+    wait_vmcnt<kBigDmaPerUnit>();
+  } else {
+    wait_vmcnt<0>();
   }
+  bare_barrier();
+  if constexpr (FMC > 0) {
+#pragma unroll
+    for (int ch = 0; ch < CH; ++ch) {
+      const char* sta = smem + (sa + xl[ch]);
+      const char* stw = smem + (sw + wl[ch]);
+#pragma unroll
+      for (int fn = 0; fn < 4; ++fn) wfP[fn][ch] = *reinterpret_cast<const uint4*>(stw + woff(fn));
+#pragma unroll
+      for (int fm = 0; fm < FMC; ++fm) xfP[fm][ch] = *reinterpret_cast<const uint4*>(sta + fm * 4096);
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#ifdef MOE_TRACE
+  const unsigned long long tr_fill = __builtin_readcyclecounter() - tr0;
+#endif
+  using Yes = IntTag<1>;
+  using No = IntTag<0>;
+  for (int kt = 0; kt + 2 < nk; ++kt) ktile(Yes{}, Yes{}, Yes{}, Yes{});
+  if (nk >= 2) ktile(Yes{}, No{}, Yes{}, No{});  // tile nk - 2: only the second half of W(nk-1) is still to come
+  ktile(No{}, No{}, No{}, No{});                  // tile nk - 1
   wait_vmcnt<0>();
 #ifdef MOE_TRACE
-  if (threadIdx.x == 0 && blockIdx.x < 4096) {
-    unsigned long long* d = moe_dbg + 8 * 4096 + 4 * 128 + blockIdx.x * 4;
-    d[0] = tr_v; d[1] = tr_b; d[2] = tr_i + 0; d[3] = __builtin_readcyclecounter() - tr0;
+  if (threadIdx.x == 0 && blockIdx.x < 16384) {
+    unsigned long long* d = moe_dbg + 8 * 16384 + blockIdx.x * 4;
+    d[0] = tr_v; d[1] = tr_b; d[2] = tr_fill; d[3] = __builtin_readcyclecounter() - tr0;
   }
 #endif
 }
@@ -676,7 +726,11 @@ __device__ __forceinline__ void big_light_mainloop(const BigCtx& c, const char* 
 #pragma unroll
     for (int i = 0; i < 2; ++i) lds_dma16(c.a_base + k * kBigRowBytes, c.a_off[i], c.dma_lds + a_slot(k) + i * 4096);
   };
-  // request order: W(0) W(1) (caller) A(0) A(1) W(2) A(2), then W(k) A(k) per K tile
+  // request order: W(0) W(1) (first half by the caller) A(0) A(1) W(2) A(2), then W(k) A(k) per K tile
+  if (1 < nk) {
+#pragma unroll
+    for (int i = 4; i < 8; ++i) lds_dma16(c.w_base + kBigRowBytes, c.w_off[i], c.dma_lds + w_slot(1) + i * 4096);
+  }
   issue_a(0);
   if (1 < nk) issue_a(1);
   if (2 < nk) { issue_w(2); issue_a(2); }
@@ -905,10 +959,13 @@ __device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, c
     for (int fm = 0; fm < 4; ++fm)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[fn][fm][r] = 0.f;
-  if constexpr (LIGHT) big_light_mainloop<Mma, FMC>(c, smem, nk, acc);
-  else big_mainloop<Mma, FMC>(c, smem, nk, acc);
+  if constexpr (LIGHT) {
+    big_light_mainloop<Mma, FMC>(c, smem, nk, acc);
+  } else {
+    big_mainloop<Mma, FMC, GATED>(c, smem, nk, acc);
+  }
 #ifdef MOE_TRACE
-  if (threadIdx.x == 0 && blockIdx.x < 4096) moe_dbg[blockIdx.x * 8 + 7] = MOE_TRACE_NOW();
+  if (threadIdx.x == 0 && blockIdx.x < 16384) moe_dbg[blockIdx.x * 8 + 7] = MOE_TRACE_NOW();
 #endif
   bare_barrier();  // every wavefront is done reading the ring before it is reused
   s_tok_all[threadIdx.x] = my_tok;
@@ -950,7 +1007,8 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
   [[maybe_unused]] const unsigned long long t_start = MOE_TRACE_NOW();
   [[maybe_unused]] const unsigned long long c_start = __builtin_readcyclecounter();
   // the two loads below do not depend on each other: one memory latency, not two
-  const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[(mb * kBigBM) / p.align_bs]);
+  int e = __builtin_amdgcn_readfirstlane(p.expert_ids[(mb * kBigBM) / p.align_bs]);
+  if (MOE_DEV_BIT(p, 2)) e = e & 1;   // dev: every tile streams the weights of two experts (hot in L2)
   const int64_t my_slot = static_cast<int64_t>(mb) * kBigBM + tid;
   const int my_tok = p.sorted_ids[my_slot < p.sorted_cap ? my_slot : p.sorted_cap - 1];
   const int n0 = nt * (GATED ? kBigBNW / 2 : kBigBNW);
@@ -984,14 +1042,14 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
     }
     c.w_off[i] = static_cast<uint32_t>(wrow * p.w_stride_n * ES + ld_chunk * 16);
   }
-  // The weights of the first two K tiles are on their way (ring slots 1 and 3) while
+  // The weights of the first K tile and a half are on their way (ring slots 1 and 3) while
   // the slot ids are still being looked at: they are the cold half of the fill.
   // Neither slot overlaps the side arrays above.
 #pragma unroll
   for (int i = 0; i < 8; ++i) lds_dma16(c.w_base, c.w_off[i], c.dma_lds + kBigUnitBytes + i * 4096);
-  if (1 < nk) {
+  if (1 < nk) {  // the first half of W(1); the main loops request the second
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < 4; ++i)
       lds_dma16(c.w_base + kBigRowBytes, c.w_off[i], c.dma_lds + 3 * kBigUnitBytes + i * 4096);
   }
   __syncthreads();
@@ -1023,7 +1081,7 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
     // groups made of padding only re-request group 0 (an L1 hit) so that every
     // token unit is exactly eight loads and the vmcnt bookkeeping stays fixed
     const int gi = i < a_groups ? i : 0;
-    const int slot = mb * kBigBM + ld_row + 32 * gi;
+    const int slot = (MOE_DEV_BIT(p, 1) ? (mb & 3) : mb) * kBigBM + ld_row + 32 * gi;   // dev bit 1: A rows of four blocks only
     int64_t src = slot;
     if (!p.a_by_slot) {
       const int tok = s_tok[ld_row + 32 * gi];
@@ -1078,7 +1136,7 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
   }
 #ifdef MOE_TRACE
   const unsigned long long t_end = MOE_TRACE_NOW();
-  if (tid == 0 && blockIdx.x < 4096) {
+  if (tid == 0 && blockIdx.x < 16384) {
     moe_dbg[blockIdx.x * 8 + 0] = t_start; moe_dbg[blockIdx.x * 8 + 1] = t_pro;
     moe_dbg[blockIdx.x * 8 + 2] = t_main; moe_dbg[blockIdx.x * 8 + 3] = t_end;
     moe_dbg[blockIdx.x * 8 + 6] = __builtin_readcyclecounter() - c_start;
@@ -1200,10 +1258,10 @@ __global__ __launch_bounds__(kThreads, 1) void big_fused_kernel(const GemmParams
 
 // Cuts the live m-blocks of a large-tile launch into one contiguous range per XCD
 // with equal estimated work instead of equal counts.  A block of an expert that
-// received at most 32 (64) rows is weight streaming only and costs about 0.56
-// (0.70) of a full one, a partly filled one 0.97 (its six gate-up and eight down
-// tiles: 318 / 394 / 542 / 562 us of CU time at 8448 tokens); with equal counts
-// the XCDs finished up to 25 % apart.
+// received at most 32 (64) rows is weight streaming only and costs about 0.60
+// (0.75) of a full one, a partly filled one as much as a full one (its six gate-up
+// and eight down tiles: 334 / 424 / 568 / 561 us of CU time at 8448 tokens); with
+// equal counts the XCDs finished up to 25 % apart.
 // Ranges stay contiguous so that the blocks of one expert keep sharing its
 // weights through one L2.  No range is longer than cap_mb blocks (the grid has
 // that many slots per XCD).  One workgroup; bounds[0..8] in m-blocks.
@@ -1222,7 +1280,7 @@ __global__ __launch_bounds__(kPlanThreads) void big_plan_kernel(const int32_t* _
   auto weight = [&](int mb) {
     if (mb >= live_mb) return 0;
     const int32_t* s = sorted_ids + static_cast<int64_t>(mb) * kBigBM;
-    return s[32] >= numel ? 36 : (s[64] >= numel ? 45 : (s[kBigBM - 1] >= numel ? 62 : 64));
+    return s[32] >= numel ? 38 : (s[64] >= numel ? 48 : 64);
   };
   // inclusive scan of `v` over the workgroup, plus the workgroup total
   auto scan = [&](int v, int& total) {
@@ -1501,7 +1559,7 @@ __global__ __launch_bounds__(kThreads, 3) void stream_gemm_kernel(const GemmPara
     }
   }
 #ifdef MOE_TRACE
-  if (tid == 0 && blockIdx.x < 4096) {
+  if (tid == 0 && blockIdx.x < 16384) {
     moe_dbg[blockIdx.x * 8 + 0] = t_start; moe_dbg[blockIdx.x * 8 + 1] = t_pro;
     moe_dbg[blockIdx.x * 8 + 2] = t_first; moe_dbg[blockIdx.x * 8 + 3] = t_loop;
     moe_dbg[blockIdx.x * 8 + 4] = MOE_TRACE_NOW(); moe_dbg[blockIdx.x * 8 + 5] = __builtin_amdgcn_s_getreg((20) | (0 << 6) | (3 << 11));
@@ -1540,6 +1598,9 @@ int launch_big(GemmParams& p, int64_t sorted_cap, hipStream_t s) {
   if (int rc = moe_opt_in_lds(opted, reinterpret_cast<const void*>(kern), lds, "fused_experts")) return rc;
   p.num_m_blocks = static_cast<int>((sorted_cap + kBigBM - 1) / kBigBM);
   p.num_n_tiles = (p.N + (GATED ? 128 : 256) - 1) / (GATED ? 128 : 256);
+#ifdef MOE_DEV
+  if (const char* f = getenv("MOE_DEV_FLAGS")) p.dev = atoi(f);
+#endif
   const int64_t tiles = static_cast<int64_t>(p.num_m_blocks) * p.num_n_tiles;
   int64_t grid = (tiles + kXcds - 1) / kXcds * kXcds;
   if (p.xcd_bounds)  // work-balanced ranges: as many slots per XCD as the longest range may have blocks
@@ -1599,6 +1660,10 @@ int launch_big_fused(GemmParams& p1, GemmParams& p2, int block_size, int64_t sor
   p2.num_n_tiles = (p2.N + 255) / 256;
   // every gate-up tile inside the matrix: its flush takes the 16-byte path, which can write through
   p1.wt_stores = (p1.N % 128 == 0 && p1.ldc % 8 == 0) ? 1 : 0;
+#ifdef MOE_DEV
+  if (const char* f = getenv("MOE_DEV_FLAGS")) p1.dev = p2.dev = atoi(f);
+  if (const char* f = getenv("MOE_DEV_FLAGS1")) p1.dev = atoi(f);
+#endif
   const int cap_mb = big_plan_cap(sorted_cap);
   const int64_t grid = static_cast<int64_t>(cap_mb) * (p1.num_n_tiles + p2.num_n_tiles) * kXcds;
   if (grid > INT32_MAX) return moe_fail(MOE_ERR_ARG, "fused_experts: grid of %lld workgroups", static_cast<long long>(grid));
