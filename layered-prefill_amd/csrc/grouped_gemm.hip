@@ -19,13 +19,6 @@
 
 #include "common.h"
 
-#ifdef MOE_TRACE
-// Development aid (make EXTRA=-DMOE_TRACE): per-workgroup phase timestamps of the large-tile kernel.
-__device__ unsigned long long moe_dbg[12 * 16384];
-#define MOE_TRACE_NOW() __builtin_amdgcn_s_memrealtime()
-#else
-#define MOE_TRACE_NOW() 0ull
-#endif
 
 namespace {
 
@@ -137,15 +130,7 @@ struct GemmParams {
   int m_major;       // workgroup order inside an XCD: all n-tiles of an m-block are neighbours
   const int32_t* xcd_bounds;  // large-tile kernel: m-block range [b[x], b[x+1]) of XCD x, or null
   int wt_stores;     // large-tile flush: results go out as device-scope write-through stores (one-launch hand-off)
-#ifdef MOE_DEV
-  int dev;           // development switches (MOE_DEV_FLAGS), never in a shipped build
-#endif
 };
-#ifdef MOE_DEV
-#define MOE_DEV_BIT(p, b) (((p).dev >> (b)) & 1)
-#else
-#define MOE_DEV_BIT(p, b) 0
-#endif
 
 constexpr int kThreads = 256;
 constexpr int kBK = 64;                  // K elements per LDS tile
@@ -556,10 +541,6 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
     wl[q] = c.w_row[0] + c.rd_k[q];
   }
   uint4 wfP[4][CH], xfP[XF][CH], wfQ[4][CH], xfQ[XF][CH];
-#ifdef MOE_TRACE
-  unsigned long long tr_v = 0, tr_b = 0;
-  const unsigned long long tr0 = __builtin_readcyclecounter();
-#endif
 
   // One MFMA step on fragment set X.  Between its MFMAs: the LDS reads of set Y (chunks of
   // MFMA step YKK of the tile whose units start at byte ya / yw of the ring) when LOAD, and
@@ -631,19 +612,9 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
       // tile kt+1 must have landed (only A(kt+2), the youngest request, may still be
       // outstanding) and nobody reads the slots of tile kt any more (its last fragment
       // reads have returned: lgkmcnt(0))
-#ifdef MOE_TRACE
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-      const unsigned long long tr1 = __builtin_readcyclecounter();
-#endif
       if constexpr (DO_A) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
       else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-#ifdef MOE_TRACE
-      const unsigned long long tr2 = __builtin_readcyclecounter();
-#endif
       bare_barrier();
-#ifdef MOE_TRACE
-      tr_v += tr2 - tr1; tr_b += __builtin_readcyclecounter() - tr2;
-#endif
       fa = sa;
       fw = sw;
       sa = next_slot(sa);
@@ -683,21 +654,12 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
     }
   }
   __builtin_amdgcn_sched_barrier(0);
-#ifdef MOE_TRACE
-  const unsigned long long tr_fill = __builtin_readcyclecounter() - tr0;
-#endif
   using Yes = IntTag<1>;
   using No = IntTag<0>;
   for (int kt = 0; kt + 2 < nk; ++kt) ktile(Yes{}, Yes{}, Yes{}, Yes{});
   if (nk >= 2) ktile(Yes{}, No{}, Yes{}, No{});  // tile nk - 2: only the second half of W(nk-1) is still to come
   ktile(No{}, No{}, No{}, No{});                  // tile nk - 1
   wait_vmcnt<0>();
-#ifdef MOE_TRACE
-  if (threadIdx.x == 0 && blockIdx.x < 16384) {
-    unsigned long long* d = moe_dbg + 8 * 16384 + blockIdx.x * 4;
-    d[0] = tr_v; d[1] = tr_b; d[2] = tr_fill; d[3] = __builtin_readcyclecounter() - tr0;
-  }
-#endif
 }
 
 // Main loop for tiles with at most 64 real slots (an expert that received only a
@@ -964,9 +926,6 @@ __device__ __forceinline__ void big_wave(const GemmParams& p, const BigCtx& c, c
   } else {
     big_mainloop<Mma, FMC, GATED>(c, smem, nk, acc);
   }
-#ifdef MOE_TRACE
-  if (threadIdx.x == 0 && blockIdx.x < 16384) moe_dbg[blockIdx.x * 8 + 7] = MOE_TRACE_NOW();
-#endif
   bare_barrier();  // every wavefront is done reading the ring before it is reused
   s_tok_all[threadIdx.x] = my_tok;
   s_rw_all[threadIdx.x] = my_rw;  // requested before the main loop, needed only now
@@ -1004,11 +963,8 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lhi = lane >> 5;
   const int wm = wave & 1, wn = wave >> 1;
-  [[maybe_unused]] const unsigned long long t_start = MOE_TRACE_NOW();
-  [[maybe_unused]] const unsigned long long c_start = __builtin_readcyclecounter();
   // the two loads below do not depend on each other: one memory latency, not two
-  int e = __builtin_amdgcn_readfirstlane(p.expert_ids[(mb * kBigBM) / p.align_bs]);
-  if (MOE_DEV_BIT(p, 2)) e = e & 1;   // dev: every tile streams the weights of two experts (hot in L2)
+  const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[(mb * kBigBM) / p.align_bs]);
   const int64_t my_slot = static_cast<int64_t>(mb) * kBigBM + tid;
   const int my_tok = p.sorted_ids[my_slot < p.sorted_cap ? my_slot : p.sorted_cap - 1];
   const int n0 = nt * (GATED ? kBigBNW / 2 : kBigBNW);
@@ -1081,7 +1037,7 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
     // groups made of padding only re-request group 0 (an L1 hit) so that every
     // token unit is exactly eight loads and the vmcnt bookkeeping stays fixed
     const int gi = i < a_groups ? i : 0;
-    const int slot = (MOE_DEV_BIT(p, 1) ? (mb & 3) : mb) * kBigBM + ld_row + 32 * gi;   // dev bit 1: A rows of four blocks only
+    const int slot = mb * kBigBM + ld_row + 32 * gi;
     int64_t src = slot;
     if (!p.a_by_slot) {
       const int tok = s_tok[ld_row + 32 * gi];
@@ -1105,7 +1061,6 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
   }
   const int slot0 = mb * kBigBM + wm * 128;
   char* epi = smem + wave * kEpiWaveBytes;
-  [[maybe_unused]] const unsigned long long t_pro = MOE_TRACE_NOW();
   const int rows = min(128, max(0, nvalid - wm * 128));  // real slots of this wavefront
   __syncthreads();  // s_tok sits inside the ring: everyone has read it before any DMA may land there
   if (nvalid <= 64) {
@@ -1123,7 +1078,6 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
     case 3: big_wave<Mma, 3, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, my_bias, s_tok, s_rw_all, epi); break;
     default: big_wave<Mma, 4, GATED>(p, c, smem, nk, e, n0, wn, wm, lane, my_tok, my_rw, my_as, my_ws, my_bias, s_tok, s_rw_all, epi); break;
   }
-  [[maybe_unused]] const unsigned long long t_main = MOE_TRACE_NOW();
   if constexpr (GATED) {
     if (p.activation == MOE_ACT_SILU)
       big_flush<El, true, MOE_ACT_SILU>(p, n0, wn, lane, slot0, rows, s_tok + wm * 128, epi);
@@ -1134,15 +1088,6 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
   } else {
     big_flush<El, false, MOE_ACT_SILU>(p, n0, wn, lane, slot0, rows, s_tok + wm * 128, epi);
   }
-#ifdef MOE_TRACE
-  const unsigned long long t_end = MOE_TRACE_NOW();
-  if (tid == 0 && blockIdx.x < 16384) {
-    moe_dbg[blockIdx.x * 8 + 0] = t_start; moe_dbg[blockIdx.x * 8 + 1] = t_pro;
-    moe_dbg[blockIdx.x * 8 + 2] = t_main; moe_dbg[blockIdx.x * 8 + 3] = t_end;
-    moe_dbg[blockIdx.x * 8 + 6] = __builtin_readcyclecounter() - c_start;
-    moe_dbg[blockIdx.x * 8 + 4] = nvalid; moe_dbg[blockIdx.x * 8 + 5] = __builtin_amdgcn_s_getreg((20) | (0 << 6) | (3 << 11));
-  }
-#endif
 }
 
 template <typename Mma, bool GATED>
@@ -1441,7 +1386,6 @@ __global__ __launch_bounds__(kThreads, 3) void stream_gemm_kernel(const GemmPara
   }
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  [[maybe_unused]] const unsigned long long t_start = MOE_TRACE_NOW();
   const int l32 = lane & 31, lhi = lane >> 5;
   const int n0 = nt * BN_OUT;
 
@@ -1511,8 +1455,6 @@ __global__ __launch_bounds__(kThreads, 3) void stream_gemm_kernel(const GemmPara
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk) rd_k[kk] = l32 * kStRowBytes + (((2 * kk + lhi) ^ ((l32 >> 1) & 7)) << 4);
 
-  [[maybe_unused]] const unsigned long long t_pro = MOE_TRACE_NOW();
-  [[maybe_unused]] unsigned long long t_first = 0;
   issue(0);
   if (1 < nu) issue(1);
   if (2 < nu) issue(2);
@@ -1523,9 +1465,6 @@ __global__ __launch_bounds__(kThreads, 3) void stream_gemm_kernel(const GemmPara
     else if (u + 1 < nu) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(kStDmaPerUnit) : "memory");
     else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     bare_barrier();
-#ifdef MOE_TRACE
-    if (u == 0) t_first = MOE_TRACE_NOW();
-#endif
     if (u + 3 < nu) issue(u + 3);
     if (wave == 0) {
       const char* st = smem + (u % kStUnits) * kStUnitBytes;
@@ -1541,7 +1480,6 @@ __global__ __launch_bounds__(kThreads, 3) void stream_gemm_kernel(const GemmPara
   }
 
   if (wave != 0) return;
-  [[maybe_unused]] const unsigned long long t_loop = MOE_TRACE_NOW();
   const int slot = mb * kStBM + l32;
   if (tok < p.numel) {
     const bool fast = n0 + BN_OUT <= p.N && (p.ldc & 3) == 0 && !p.w_scale;
@@ -1558,13 +1496,6 @@ __global__ __launch_bounds__(kThreads, 3) void stream_gemm_kernel(const GemmPara
       store_fragment<El, false>(p, e, acc1, acc1, tok, slot, n0 + 32 + 4 * lhi, rw);
     }
   }
-#ifdef MOE_TRACE
-  if (tid == 0 && blockIdx.x < 16384) {
-    moe_dbg[blockIdx.x * 8 + 0] = t_start; moe_dbg[blockIdx.x * 8 + 1] = t_pro;
-    moe_dbg[blockIdx.x * 8 + 2] = t_first; moe_dbg[blockIdx.x * 8 + 3] = t_loop;
-    moe_dbg[blockIdx.x * 8 + 4] = MOE_TRACE_NOW(); moe_dbg[blockIdx.x * 8 + 5] = __builtin_amdgcn_s_getreg((20) | (0 << 6) | (3 << 11));
-  }
-#endif
 }
 
 template <typename Mma, bool GATED>
@@ -1598,9 +1529,6 @@ int launch_big(GemmParams& p, int64_t sorted_cap, hipStream_t s) {
   if (int rc = moe_opt_in_lds(opted, reinterpret_cast<const void*>(kern), lds, "fused_experts")) return rc;
   p.num_m_blocks = static_cast<int>((sorted_cap + kBigBM - 1) / kBigBM);
   p.num_n_tiles = (p.N + (GATED ? 128 : 256) - 1) / (GATED ? 128 : 256);
-#ifdef MOE_DEV
-  if (const char* f = getenv("MOE_DEV_FLAGS")) p.dev = atoi(f);
-#endif
   const int64_t tiles = static_cast<int64_t>(p.num_m_blocks) * p.num_n_tiles;
   int64_t grid = (tiles + kXcds - 1) / kXcds * kXcds;
   if (p.xcd_bounds)  // work-balanced ranges: as many slots per XCD as the longest range may have blocks
@@ -1660,10 +1588,6 @@ int launch_big_fused(GemmParams& p1, GemmParams& p2, int block_size, int64_t sor
   p2.num_n_tiles = (p2.N + 255) / 256;
   // every gate-up tile inside the matrix: its flush takes the 16-byte path, which can write through
   p1.wt_stores = (p1.N % 128 == 0 && p1.ldc % 8 == 0) ? 1 : 0;
-#ifdef MOE_DEV
-  if (const char* f = getenv("MOE_DEV_FLAGS")) p1.dev = p2.dev = atoi(f);
-  if (const char* f = getenv("MOE_DEV_FLAGS1")) p1.dev = atoi(f);
-#endif
   const int cap_mb = big_plan_cap(sorted_cap);
   const int64_t grid = static_cast<int64_t>(cap_mb) * (p1.num_n_tiles + p2.num_n_tiles) * kXcds;
   if (grid > INT32_MAX) return moe_fail(MOE_ERR_ARG, "fused_experts: grid of %lld workgroups", static_cast<long long>(grid));
@@ -1966,8 +1890,3 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   return moe_sum(a->out, c3, a->T, a->K, a->H, a->act_dtype, a->stream);
 }
 
-#ifdef MOE_TRACE
-MOE_EXPORT int moe_debug_read(void* dst, int64_t bytes) {
-  return hipMemcpyFromSymbol(dst, HIP_SYMBOL(moe_dbg), bytes) == hipSuccess ? 0 : -1;
-}
-#endif

@@ -11,18 +11,12 @@ import torch
 from . import _lib
 from ._lib import check, lib, require_gpu_tensor, stream_ptr
 
-# scratch for the three-launch alignment path, one buffer per (device, stream)
-# so that concurrent streams never share it; grown on demand, never shrunk
-_align_ws: dict = {}
-
-
 def _align_workspace(nbytes: int, device: torch.device) -> torch.Tensor:
-    key = (device.index, stream_ptr(device))
-    buf = _align_ws.get(key)
-    if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(nbytes, 1 << 16), dtype=torch.uint8, device=device)
-        _align_ws[key] = buf
-    return buf
+    """Scratch for the three-launch alignment path, taken from torch's caching
+    allocator on every call: the block is tied to the current stream, which is
+    the stream the kernels are enqueued on, so its reuse after the call is
+    ordered behind them and nothing outlives the call."""
+    return torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
 
 
 def topk_softmax(topk_weights: torch.Tensor, topk_indices: torch.Tensor,
