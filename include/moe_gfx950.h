@@ -55,7 +55,9 @@ int moe_abi_version(void);
  * topk_weights[T,K] (softmax values, or those divided by their sum over k when
  * renormalize != 0, which is nanovllm/layers/for_moe/fused_moe.py:417-418),
  * topk_ids[T,K] and token_expert_indices[T,K] = k*T + row.  Needs no
- * workspace for any E in [1, 1024]; requires K <= E. */
+ * workspace for any E in [1, 16384] (a row beyond 1024 columns is kept in LDS
+ * by the one wavefront that owns it; MOE_ERR_UNSUPPORTED above 16384);
+ * requires K <= E. */
 int moe_topk_softmax(const float* gating_output, float* topk_weights, int32_t* topk_ids,
                      int32_t* token_expert_indices, int T, int E, int K, int renormalize,
                      void* stream);

@@ -6,7 +6,7 @@
 // the same column-to-lane assignment and the same butterfly order, as in the
 // reference's fused kernel, so the fp32 sum has the same association; the
 // 64-lane wavefront simply carries twice as many rows as a 32-lane warp.
-// Any other E <= 1024 takes one wavefront per row.
+// Any other E takes one wavefront per row: in registers up to 1024 columns, in LDS up to 16384.
 #include <stdarg.h>
 
 #include "common.h"
@@ -456,6 +456,68 @@ __global__ __launch_bounds__(kWave* kWavesPerBlock) void topk_softmax_generic_ke
   }
 }
 
+// Wider rows (more columns than 64 lanes x 16 registers): one wavefront per row,
+// the row's probabilities in LDS.  Lane l owns columns l, l+64, ... exactly as in
+// the register kernel above, so the order of every max, sum and comparison is the
+// same; every LDS word is read and written by its owning lane only, which is why
+// no barrier appears.
+constexpr int kWideMaxExperts = 16384;  // 64 KiB of LDS per row
+
+__global__ __launch_bounds__(kWave) void topk_softmax_wide_kernel(
+    const float* __restrict__ gating, float* __restrict__ topk_w, int32_t* __restrict__ topk_ids,
+    int32_t* __restrict__ tok_exp_idx, int T, int E, int K, int renormalize) {
+  extern __shared__ float prob[];
+  const int lane = threadIdx.x;
+  const int row = blockIdx.x;
+  const float* src = gating + static_cast<size_t>(row) * E;
+  const float ninf = -__builtin_inff();
+
+  float mx = ninf;
+  for (int c = lane; c < E; c += kWave) mx = fmaxf(mx, src[c]);
+#pragma unroll
+  for (int m = 32; m > 0; m /= 2) mx = fmaxf(mx, __shfl_xor(mx, m, kWave));
+  float sum = 0.f;
+  for (int c = lane; c < E; c += kWave) {
+    const float e = moe_expf(src[c] - mx);
+    prob[c] = e;
+    sum += e;
+  }
+#pragma unroll
+  for (int m = 32; m > 0; m /= 2) sum += __shfl_xor(sum, m, kWave);
+  const float rinv = 1.f / sum;
+  for (int c = lane; c < E; c += kWave) prob[c] = prob[c] * rinv;
+
+  float wsum = 0.f;
+  for (int k = 0; k < K; ++k) {
+    float best = -20000.f;  // below the marker of a taken column
+    int bidx = lane;
+    for (int c = lane; c < E; c += kWave) {
+      const float v = prob[c];
+      if (v > best) { best = v; bidx = c; }
+    }
+#pragma unroll
+    for (int m = 32; m > 0; m /= 2) {
+      float ov = __shfl_xor(best, m, kWave);
+      int oi = __shfl_xor(bidx, m, kWave);
+      if (ov > best || (ov == best && oi < bidx)) { best = ov; bidx = oi; }
+    }
+    if (lane == 0) {
+      const size_t o = static_cast<size_t>(row) * K + k;
+      topk_w[o] = best;
+      topk_ids[o] = bidx;
+      tok_exp_idx[o] = k * T + row;
+    }
+    wsum += best;
+    if (lane == bidx % kWave) prob[bidx] = -10000.f;
+  }
+  if (renormalize && lane == 0) {
+    for (int k = 0; k < K; ++k) {
+      const size_t o = static_cast<size_t>(row) * K + k;
+      topk_w[o] = topk_w[o] / wsum;
+    }
+  }
+}
+
 template <int E>
 void launch_pow2(const float* g, float* w, int32_t* ids, int32_t* tei, int T, int K, int renorm,
                  hipStream_t s) {
@@ -472,8 +534,8 @@ MOE_EXPORT int moe_topk_softmax(const float* gating_output, float* topk_weights,
                                 int renormalize, void* stream) {
   if (T < 0 || E < 1 || K < 1) return moe_fail(MOE_ERR_ARG, "topk_softmax: bad sizes T=%d E=%d K=%d", T, E, K);
   if (K > E) return moe_fail(MOE_ERR_ARG, "topk_softmax: topk %d exceeds num_experts %d", K, E);
-  if (E > kWave * kGenericMaxPerLane)
-    return moe_fail(MOE_ERR_UNSUPPORTED, "topk_softmax: num_experts %d > %d", E, kWave * kGenericMaxPerLane);
+  if (E > kWideMaxExperts)
+    return moe_fail(MOE_ERR_UNSUPPORTED, "topk_softmax: num_experts %d > %d", E, kWideMaxExperts);
   if (static_cast<int64_t>(T) * K > INT32_MAX)
     return moe_fail(MOE_ERR_ARG, "topk_softmax: T*K overflows int32 token_expert_indices");
   if (T == 0) return MOE_OK;
@@ -491,6 +553,12 @@ MOE_EXPORT int moe_topk_softmax(const float* gating_output, float* topk_weights,
     case 128: launch_pow2<128>(gating_output, topk_weights, topk_ids, token_expert_indices, T, K, renormalize, s); break;
     case 256: launch_pow2<256>(gating_output, topk_weights, topk_ids, token_expert_indices, T, K, renormalize, s); break;
     default: {
+      if (E > kWave * kGenericMaxPerLane) {
+        hipLaunchKernelGGL(topk_softmax_wide_kernel, dim3(T), dim3(kWave), sizeof(float) * E, s,
+                           gating_output, topk_weights, topk_ids, token_expert_indices, T, E, K,
+                           renormalize);
+        break;
+      }
       const int blocks = (T + kWavesPerBlock - 1) / kWavesPerBlock;
       hipLaunchKernelGGL(topk_softmax_generic_kernel, dim3(blocks), dim3(kWave * kWavesPerBlock), 0,
                          s, gating_output, topk_weights, topk_ids, token_expert_indices, T, E, K,

@@ -16,7 +16,8 @@ def _run_topk(moe, g, K, renorm, dev):
     return w.cpu(), ids.cpu(), tei.cpu()
 
 
-@pytest.mark.parametrize("E", [1, 2, 4, 8, 16, 32, 64, 128, 256, 3, 48, 100, 384, 1000, 1024])
+@pytest.mark.parametrize("E", [1, 2, 4, 8, 16, 32, 64, 128, 256, 3, 48, 100, 384, 1000, 1024,
+                               1025, 1500, 2048, 5000, 16384])
 @pytest.mark.parametrize("T", [1, 7, 257])
 def test_topk_softmax_bit_exact(moe, oracle, dev, E, T):
     print(f"topk_softmax E={E} T={T}", flush=True)
@@ -28,6 +29,27 @@ def test_topk_softmax_bit_exact(moe, oracle, dev, E, T):
             assert torch.equal(ids, oids), (E, T, K, renorm)
             assert torch.equal(tei, otei)
             assert torch.equal(w.view(torch.int32), ow.view(torch.int32)), (E, T, K, renorm)
+
+
+def test_topk_softmax_wide_rows_ties_subnormals_and_limit(moe, oracle, dev):
+    """Rows of more than 1024 columns (the reference's fallback takes any E,
+    csrc/moe_topk_softmax_kernels.cu:460-469): equal logits pick the lowest
+    indices, a spread that reaches subnormal probabilities ranks as the oracle
+    does, and the first unsupported width fails with a message."""
+    E = 3000
+    g = torch.zeros(5, E)
+    w, ids, _ = _run_topk(moe, g, 8, False, dev)
+    assert torch.equal(ids, torch.arange(8, dtype=torch.int32).repeat(5, 1))
+    gen = torch.Generator().manual_seed(77)
+    x = -(torch.rand(33, E, generator=gen) * 40 + 80)
+    x[torch.arange(33), torch.randint(0, E, (33,), generator=gen)] = 0.0
+    for renorm in (False, True):
+        w, ids, tei = _run_topk(moe, x, 16, renorm, dev)
+        ow, oids, otei = oracle.topk_softmax(x, 16, renormalize=renorm)
+        assert torch.equal(ids, oids) and torch.equal(tei, otei)
+        assert torch.equal(w.view(torch.int32), ow.view(torch.int32))
+    with pytest.raises(RuntimeError, match="num_experts 16385"):
+        _run_topk(moe, torch.zeros(2, 16385), 2, False, dev)
 
 
 def test_topk_softmax_ties_and_bf16_logits(moe, oracle, dev):
