@@ -74,7 +74,7 @@ def _softmax64(g):
 
 @pytest.mark.parametrize("E,K", [(1, 1), (2, 1), (4, 2), (8, 2), (16, 4), (32, 8), (64, 6),
                                  (128, 8), (256, 8), (3, 2), (48, 4), (100, 8), (384, 8),
-                                 (1000, 5)])
+                                 (1000, 5), (1025, 8), (5000, 16)])
 def test_topk_softmax_against_float64_softmax(oracle, E, K):
     g = torch.randn(37, E, generator=torch.Generator().manual_seed(E * 31 + K))
     w, ids, tei, probs = oracle.topk_softmax(g, K, return_probs=True)
