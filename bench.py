@@ -298,6 +298,43 @@ def time_stages(layer: Layer, steps: int, warmup: int = 10):
     return {n: statistics.fmean(v) for n, v in per.items()}, ids
 
 
+def balanced_routing(moe, layer: "Layer", steps: int, warmup: int):
+    """The same layer with every expert receiving the same number of rows: the first
+    7936 tokens, token t's choice k going to expert (37 * (K t + k)) mod E with weight
+    1/K, which at E = 128, K = 8 gives every expert 496 rows: one full 256-slot block and
+    one of 240 rows, and no workgroup left streaming the weights of an expert with a
+    handful of rows.  (7936 rather than 8192 tokens so that the launch has a grid of its
+    own in a kernel trace.)  Routing and alignment are timed with it, as in the headline
+    step.  The number says how much of the headline's distance to the peak is the
+    benchmark routing's skew and how much is the kernels'."""
+    s = layer.shape
+    K, E = s.top_k, s.experts
+    T = min(layer.T, 7936)
+    x, logits = layer.x[:T].contiguous(), layer.logits[:T].contiguous()
+    t = torch.arange(T, device=layer.dev).view(T, 1)
+    k = torch.arange(K, device=layer.dev).view(1, K)
+    ids = ((t * K + k) * 37 % E).to(torch.int32).contiguous()
+    tw = torch.full((T, K), 1.0 / K, dtype=torch.float32, device=layer.dev)
+    counts = torch.bincount(ids.flatten().long(), minlength=E)
+
+    def step():
+        moe.fused_topk(x, logits, K, True)          # timed like the headline, result unused
+        return moe.fused_experts(x, layer.w13, layer.w2, None, None, tw, ids)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    fl = moe.workloads.layer_flops(T, s)
+    return {"tokens": T, "rows_per_expert": [int(counts.min()), int(counts.max())], "ms_per_step": round(ms, 4),
+            "tflops": round(fl / (ms * 1e-3) / 1e12, 2),
+            "frac_of_bf16_peak": round(fl / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4)}
+
+
 def chunk_amplification(moe, layer: "Layer", reps: int, mode: str = "both"):
     """Config 4: the 8192-token prompt as 16 chunks of 512 tokens, each co-batched
     with the 256 decode tokens (16 calls of T=768), against the single 8192+256
@@ -405,6 +442,8 @@ def legs(a, moe, dev, wl, main_layer, shape, flops, out) -> None:
     out["router_gate"] = time_router_gate(moe, main_layer, 50)
     if compute_bound and not a.no_trace_mix:
         out["trace_mix"] = trace_mix(moe, main_layer, max(10, a.steps // 4))
+    if compute_bound and not a.no_balanced:
+        out["balanced_routing"] = balanced_routing(moe, main_layer, max(10, a.steps // 4), max(5, a.warmup // 2))
     if compute_bound and a.chunk_mode != "off":
         out["chunk_amplification"] = chunk_amplification(moe, main_layer, max(2, a.steps // 10), a.chunk_mode)
     if compute_bound and not a.no_fp8:
@@ -451,6 +490,7 @@ def main() -> int:
                          "rocprofv3 counter runs), or off")
     ap.add_argument("--no-fp8", action="store_true", help="skip the e4m3 leg (config 5)")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay of the decode leg")
+    ap.add_argument("--no-balanced", action="store_true", help="skip the balanced-routing leg")
     ap.add_argument("--no-trace-mix", action="store_true",
                     help="skip the layered-prefill call-size mix of the ShareGPT length sample")
     ap.add_argument("--copy-calibration", action="store_true",
