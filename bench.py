@@ -442,10 +442,10 @@ def legs(a, moe, dev, wl, main_layer, shape, flops, out) -> None:
     out["router_gate"] = time_router_gate(moe, main_layer, 50)
     if compute_bound and not a.no_trace_mix:
         out["trace_mix"] = trace_mix(moe, main_layer, max(10, a.steps // 4))
-    if compute_bound and not a.no_balanced:
-        out["balanced_routing"] = balanced_routing(moe, main_layer, max(10, a.steps // 4), max(5, a.warmup // 2))
     if compute_bound and a.chunk_mode != "off":
         out["chunk_amplification"] = chunk_amplification(moe, main_layer, max(2, a.steps // 10), a.chunk_mode)
+    if compute_bound and not a.no_balanced:
+        out["balanced_routing"] = balanced_routing(moe, main_layer, max(20, a.steps // 4), max(20, a.warmup // 2))
     if compute_bound and not a.no_fp8:
         # config 5: e4m3 weights (per-output-channel scales), per-token e4m3 activations
         w13q, w13s, w2q, w2s = moe.quantize_expert_weights(main_layer.w13, main_layer.w2)
