@@ -361,7 +361,7 @@ def fused_experts_impl(hidden_states: torch.Tensor,
                                     expert_ids, num_tokens_post_padded, bm, activation,
                                     apply_router_weight_on_input, weight_code=weight_code,
                                     workspace=workspace, passes=16 if plan is not None else 0)
-        if _CHECK_HANDOFF:
+        if _CHECK_HANDOFF and not torch.cuda.is_current_stream_capturing():  # the check waits for the stream
             fused_experts_status(args)
     return out_hidden_states
 
