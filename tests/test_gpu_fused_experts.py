@@ -476,6 +476,37 @@ def test_large_tile_ranges_on_lopsided_routing(moe, oracle, dev, pattern, monkey
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("rows_per_expert", [256, 512, 32, 255, 257])
+def test_experts_with_exactly_full_blocks(moe, oracle, dev, rows_per_expert):
+    """Every expert receives the same number of rows: exact multiples of the 256-slot block
+    (no padding slot anywhere: the padded total equals the number of routed rows), of the
+    32-slot block, and one row to either side of a block boundary."""
+    E, H, I, K = 16, 256, 128, 2
+    T = rows_per_expert * E // K
+    g = torch.Generator().manual_seed(5 + rows_per_expert)
+    t = torch.arange(T).view(T, 1)
+    k = torch.arange(K).view(1, K)
+    ids = ((t * K + k) * 5 % E).to(torch.int32)            # 5 and E coprime: every expert T K / E rows
+    assert torch.bincount(ids.flatten().long(), minlength=E).unique().tolist() == [rows_per_expert]
+    x = torch.randn(T, H, generator=g).bfloat16()
+    w13 = (torch.randn(E, 2 * I, H, generator=g) * 0.05).bfloat16()
+    w2 = (torch.randn(E, H, I, generator=g) * 0.05).bfloat16()
+    tw = torch.rand(T, K, generator=g) + 0.5
+    d = lambda z: z.to(dev)
+    for bm in (256, 32):
+        so, eo, npp = moe.fused_moe.moe_align_block_size(d(ids), bm, E)
+        oso, oeo, onpp = oracle.moe_align_block_size(ids, bm, E)
+        assert torch.equal(so.cpu(), oso) and torch.equal(eo.cpu(), oeo) and int(npp) == int(onpp)
+        if rows_per_expert % bm == 0:
+            assert int(npp) == T * K
+        out = torch.empty(T, H, dtype=torch.bfloat16, device=dev)
+        moe.fused_moe.launch_fused_experts(d(x), out, d(w13), d(w2), None, None, None, None, d(tw), so, eo, npp, bm)
+        mode = _mode(moe, T, E, K, H, torch.bfloat16, bm=bm)
+        _close_mirrored(out, lambda m: oracle.fused_experts_ref(x, w13, w2, tw, ids, mirror_rounding=m), mode,
+                        rtol=1.6e-2, atol=2e-3 + 4e-3 * out.float().abs().max().item())
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("E,H,I,T,K,act", [(16, 512, 256, 2500, 4, "silu"), (8, 256, 192, 3000, 2, "swigluoai"),
                                           (64, 256, 128, 6000, 8, "silu")])
