@@ -477,7 +477,8 @@ static int align_impl(const void* topk_ids, int ids_dtype, int64_t numel, int E,
     return moe_fail(MOE_ERR_ARG, "moe_align_block_size: expert_ids holds %lld, needs %lld",
                     static_cast<long long>(expert_cap),
                     static_cast<long long>((need_sorted + block_size - 1) / block_size));
-  if (!sorted_token_ids || !expert_ids || !num_tokens_post_pad || (numel > 0 && !topk_ids))
+  // (an empty output - no ids and blocks of one slot - may come with a null pointer)
+  if ((need_sorted > 0 && (!sorted_token_ids || !expert_ids)) || !num_tokens_post_pad || (numel > 0 && !topk_ids))
     return moe_fail(MOE_ERR_ARG, "moe_align_block_size: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int id_bits = bits_for(E);

@@ -121,7 +121,7 @@ def test_topk_softmax_rejects_bad_arguments(moe, dev):
 
 # ------------------------------------------------------------------ alignment
 ALIGN_CASES = [
-    (0, 8, 16), (1, 1, 1), (9, 5, 4), (12, 5, 4), (128, 8, 64), (2048, 128, 16), (2048, 128, 32),
+    (0, 8, 16), (0, 8, 1), (1, 1, 1), (9, 5, 4), (12, 5, 4), (128, 8, 64), (2048, 128, 16), (2048, 128, 32),
     (2048, 128, 64), (2048, 128, 128), (6144, 128, 64), (16384, 128, 32), (16385, 128, 32),
     (67584, 128, 64), (67584, 128, 128), (67584, 128, 16), (524288, 128, 128), (30000, 60, 7),
     (5000, 1000, 16), (70000, 1024, 8), (3000, 600, 32), (40000, 512, 64), (1000, 2, 256),
