@@ -121,5 +121,10 @@ __device__ __forceinline__ float moe_swigluoai(float g, float u, float alpha, fl
   float cu = u > limit ? limit : (u < -limit ? -limit : u);
   float sig = 1.0f / (1.0f + moe_expf(-cg * alpha));
   float glu = cg * sig;
-  return (cu + 1.0f) * glu;
+  float r = (cu + 1.0f) * glu;
+  // The product is an fp32 value before it is narrowed, as in the reference's kernel.  Without
+  // this the compiler may fold the multiplication into the conversion to fp16 (one rounding
+  // of the exact product instead of two), which differs in one element in ten thousand.
+  asm volatile("" : "+v"(r));
+  return r;
 }

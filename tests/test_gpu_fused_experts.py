@@ -203,10 +203,14 @@ def test_silu_and_mul_bit_exact(moe, oracle, dev, dtype, rows, d):
                        want.view(torch.int16 if dtype != torch.float32 else torch.int32))
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_swigluoai_and_mul_bit_exact(moe, oracle, dev, dtype):
-    x = (torch.randn(40, 2 * 360, generator=torch.Generator().manual_seed(1)) * 5).to(dtype)
-    out = torch.empty(40, 360, dtype=dtype, device=dev)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,d", [(40, 360), (5000, 7), (3000, 1)])
+def test_swigluoai_and_mul_bit_exact(moe, oracle, dev, dtype, rows, d):
+    """Vector path (d a multiple of 8) and element path.  fp16 with many rows is the case in
+    which a multiplication folded into the narrowing conversion (one rounding instead of
+    two) shows: about one element in ten thousand."""
+    x = (torch.randn(rows, 2 * d, generator=torch.Generator().manual_seed(1)) * 3).to(dtype)
+    out = torch.empty(rows, d, dtype=dtype, device=dev)
     moe.ops.swigluoai_and_mul(out, x.to(dev), 1.702, 7.0)
     want = oracle.swigluoai_and_mul(x, 1.702, 7.0)
     assert torch.equal(out.cpu().view(torch.int16 if dtype != torch.float32 else torch.int32),
