@@ -7,15 +7,17 @@
  *  - Every pointer is a device pointer on the current HIP device unless its
  *    name says otherwise.  The library borrows them for the enqueued work
  *    only; it never allocates, frees or retains device memory, never
- *    synchronises the device and never copies device -> host.  All launch
- *    dimensions come from upper bounds known on the host, so each call can be
- *    recorded into a HIP graph.
+ *    synchronises the device and never copies device -> host (one exception,
+ *    named as such below: moe_fused_experts_status waits for the stream and
+ *    reads one word back).  All launch dimensions come from upper bounds known
+ *    on the host, so each call can be recorded into a HIP graph.
  *  - `stream` is a hipStream_t passed as void* (NULL = the null stream).
  *  - Return value 0 = enqueued; negative = rejected, nothing enqueued.
  *    `moe_last_error()` then returns a thread-local, human-readable reason.
- *  - Host-side state: the per-device "large LDS opted in" flags of the kernels and the
- *    wait limit of moe_fused_experts_set_wait_limit, all atomics; entry points may be
- *    called from several host threads.
+ *  - Host-side state: the per-device "large LDS opted in" flags of the kernels, the
+ *    wait limit of moe_fused_experts_set_wait_limit and the per-device address of the
+ *    built-in scratch array of moe_align_block_size_static, all atomics; entry points
+ *    may be called from several host threads.
  *  - Scratch memory comes from the caller (`workspace`), sized by the
  *    matching `*_workspace_bytes` function, 256-byte aligned.
  */
