@@ -74,14 +74,26 @@ class Layer:
     """Inputs of one workload on the GPU plus the pre-allocated scratch a
     serving loop would reuse."""
 
-    def __init__(self, moe, name: str, dev):
+    def __init__(self, moe, name: str, dev, layout: str = "plain", weights=None):
+        """``layout`` "tiled": the expert weights the steps run on are the copies that
+        ``FusedMoE.process_weights_after_loading`` makes once after loading
+        (``ops.tile_expert_weights``); ``w13`` / ``w2`` stay the row-major tensors.
+        ``weights``: (w13, w2, w13_run, w2_run) of another Layer of the same model, shared."""
         wl = moe.workloads
         self.moe = moe
         self.name = name
         self.shape, x, logits, w13, w2 = wl.make_config(name)
         self.T = x.shape[0]
         self.x, self.logits = x.to(dev), logits.to(dev)
-        self.w13, self.w2 = w13.to(dev), w2.to(dev)
+        self.layout = layout
+        if weights is not None:
+            self.w13, self.w2, self.w13_run, self.w2_run = weights
+        else:
+            self.w13, self.w2 = w13.to(dev), w2.to(dev)
+            self.w13_run, self.w2_run = self.w13, self.w2
+            if layout == "tiled":
+                self.w13_run = moe.ops.tile_expert_weights(self.w13, True)
+                self.w2_run = moe.ops.tile_expert_weights(self.w2, False)
         self.dev = dev
         s = self.shape
         self.bm = moe.try_get_optimal_moe_config(self.w13.shape, self.w2.shape, s.top_k, None,
@@ -91,10 +103,26 @@ class Layer:
         self.workspace = torch.empty(ws, dtype=torch.uint8, device=dev)
         self.out = torch.empty_like(self.x)
 
+    def experts(self, x, tw, ids):
+        """``fused_experts`` on this layer's weights in the layout it runs with."""
+        return self.moe.fused_experts(x, self.w13_run, self.w2_run, None, None, tw, ids, weight_layout=self.layout)
+
+    def with_layout(self, layout: str) -> "Layer":
+        """The same inputs, weights and scratch run with the other weight layout."""
+        other = Layer.__new__(Layer)
+        other.__dict__.update(self.__dict__)
+        other.layout = layout
+        if layout == "plain":
+            other.w13_run, other.w2_run = self.w13, self.w2
+        elif self.layout != "tiled":
+            other.w13_run = self.moe.ops.tile_expert_weights(self.w13, True)
+            other.w2_run = self.moe.ops.tile_expert_weights(self.w2, False)
+        return other
+
     def step(self):
         moe, s = self.moe, self.shape
         tw, ids, _ = moe.fused_topk(self.x, self.logits, s.top_k, True)
-        return moe.fused_experts(self.x, self.w13, self.w2, None, None, tw, ids)
+        return self.experts(self.x, tw, ids)
 
     def step_instrumented(self, ev):
         """Same work with an event after every stage (5 stages -> 6 events), the two
@@ -109,13 +137,14 @@ class Layer:
         sorted_ids, expert_ids, npp = fm.moe_align_block_size(ids, self.bm, s.experts)
         ev[2].record()
         for i, mask in enumerate((1, 2, 4)):
-            fm.launch_fused_experts(self.x, self.out, self.w13, self.w2, None, None, None, None, tw,
+            fm.launch_fused_experts(self.x, self.out, self.w13_run, self.w2_run, None, None, None, None, tw,
                                     sorted_ids, expert_ids, npp, self.bm, workspace=self.workspace,
-                                    passes=mask)
+                                    passes=mask, weight_layout=self.layout)
             ev[3 + i].record()
         ev[6].record()
-        fm.launch_fused_experts(self.x, self.out, self.w13, self.w2, None, None, None, None, tw,
-                                sorted_ids, expert_ids, npp, self.bm, workspace=self.workspace, passes=3)
+        fm.launch_fused_experts(self.x, self.out, self.w13_run, self.w2_run, None, None, None, None, tw,
+                                sorted_ids, expert_ids, npp, self.bm, workspace=self.workspace, passes=3,
+                                weight_layout=self.layout)
         ev[7].record()
         return ids
 
@@ -132,6 +161,32 @@ def time_steps(layer: Layer, steps: int, warmup: int):
         layer.step()
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def time_steps_rotating(layer: Layer, steps: int, warmup: int, nsets: int = 4):
+    """Back-to-back steps, no host synchronisation, each on the next of ``nsets`` distinct
+    copies of the expert weights (the experts rotated by one per copy, so every copy is a
+    different 1.2 GB in memory: 4.8 GB in all against 256 MB of memory-side cache).  A step
+    then finds none of its weights in any cache, as in a model whose layers each bring their
+    own experts, while the GPU stays in the sustained state of the timed loop."""
+    sets = [(layer.w13_run.roll(k, 0).contiguous(), layer.w2_run.roll(k, 0).contiguous()) for k in range(nsets)]
+    moe, s = layer.moe, layer.shape
+
+    def step(i):
+        tw, ids, _ = moe.fused_topk(layer.x, layer.logits, s.top_k, True)
+        w13, w2 = sets[i % nsets]
+        return moe.fused_experts(layer.x, w13, w2, None, None, tw, ids, weight_layout=layer.layout)
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    del sets
+    return ms
 
 
 def time_steps_flushed(layer: Layer, steps: int):
@@ -253,7 +308,7 @@ def trace_mix(moe, layer: Layer, steps: int):
 
         def step():
             tw, ids, _ = moe.fused_topk(x, logits, s.top_k, True)
-            return moe.fused_experts(x, layer.w13, layer.w2, None, None, tw, ids)
+            return layer.experts(x, tw, ids)
 
         # sustained rate per bucket: about 40 ms of warm-up, then `steps` timed calls
         for _ in range(max(3, min(200, int(40.0 / (0.1 + b * 1e-4))))):
@@ -321,7 +376,7 @@ def balanced_routing(moe, layer: "Layer", steps: int, warmup: int):
 
     def step():
         moe.fused_topk(x, logits, K, True)          # timed like the headline, result unused
-        return moe.fused_experts(x, layer.w13, layer.w2, None, None, tw, ids)
+        return layer.experts(x, tw, ids)
 
     for _ in range(warmup):
         step()
@@ -353,7 +408,7 @@ def chunk_amplification(moe, layer: "Layer", reps: int, mode: str = "both"):
         act = 0
         for xc, lc in chunks:
             tw, ids, _ = moe.fused_topk(xc, lc, s.top_k, True)
-            moe.fused_experts(xc, layer.w13, layer.w2, None, None, tw, ids)
+            layer.experts(xc, tw, ids)
         return act
 
     def timed(fn):
@@ -419,7 +474,7 @@ def legs(a, moe, dev, wl, main_layer, shape, flops, out) -> None:
     # function then start from the clocks and power state of sustained large calls, not from the
     # low-power state the decode-sized legs leave behind
     if compute_bound:
-        dec = Layer(moe, "decode_256", dev)
+        dec = Layer(moe, "decode_256", dev, a.weight_layout)
         dms = time_steps(dec, max(a.steps, 50), max(a.warmup, 10))
         dstages, dids = time_stages(dec, 20)
         dact = dec.n_active(dids)
@@ -429,6 +484,15 @@ def legs(a, moe, dev, wl, main_layer, shape, flops, out) -> None:
                          "hbm_gbs": round(dgbs, 1), "frac_of_hbm_peak": round(dgbs / PEAK_HBM_GBS, 4),
                          "active_experts": dact, "block_size_m": dec.bm,
                          "stage_ms": {k: round(v, 4) for k, v in dstages.items()}}
+        rms = time_steps_rotating(dec, max(a.steps, 60), max(a.warmup, 12))
+        out["decode"]["rotating_weights"] = {"weight_sets": 4, "ms_per_step": round(rms, 4),
+                                             "hbm_gbs": round(dbytes / (rms * 1e-3) / 1e9, 1),
+                                             "frac_of_hbm_peak": round(dbytes / (rms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+        if a.weight_layout != "plain":
+            pms = time_steps(dec.with_layout("plain"), max(a.steps, 50), max(a.warmup, 10))
+            out["decode"]["plain_layout"] = {"ms_per_step": round(pms, 4),
+                                             "hbm_gbs": round(dbytes / (pms * 1e-3) / 1e9, 1),
+                                             "frac_of_hbm_peak": round(dbytes / (pms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
         out["decode"]["router_gate"] = time_router_gate(moe, dec, 100)
         fmed, fp10, fp90 = time_steps_flushed(dec, 30)
         out["decode"]["cache_flushed"] = {"ms_median": round(fmed, 4), "ms_p10": round(fp10, 4),
@@ -505,6 +569,10 @@ def main() -> int:
                          "FETCH_SIZE / WRITE_SIZE readings are scaled by")
     ap.add_argument("--only-chunk-leg", action="store_true",
                     help="run nothing but the chunk-amplification leg")
+    ap.add_argument("--weight-layout", default="tiled", choices=["tiled", "plain"],
+                    help="expert weights as FusedMoE(weight_layout=...).process_weights_after_loading leaves "
+                         "them: re-ordered once into the DMA kernels' unit order (tiled), or row-major as "
+                         "loaded (plain; with tiled, the plain figures are reported next to it)")
     ap.add_argument("--block-size-m", type=int, default=0,
                     help="override the alignment block size (0 = the library's choice)")
     a = ap.parse_args()
@@ -530,7 +598,7 @@ def main() -> int:
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    main_layer = Layer(moe, a.workload, dev)
+    main_layer = Layer(moe, a.workload, dev, a.weight_layout)
     if a.only_chunk_leg:
         print(json.dumps({"chunk_amplification": chunk_amplification(moe, main_layer, max(2, a.steps // 10),
                                                                       a.chunk_mode)}))
@@ -545,6 +613,8 @@ def main() -> int:
     out = {}
     legs(a, moe, dev, wl, main_layer, shape, flops, out)
     ms = time_steps(main_layer, a.steps, a.warmup)
+    ms_plain = time_steps(main_layer.with_layout("plain"), a.steps, a.warmup) if a.weight_layout != "plain" else None
+    ms_rot = time_steps_rotating(main_layer, a.steps, a.warmup)
     stages, ids = time_stages(main_layer, max(5, a.steps // 2))
     n_active = main_layer.n_active(ids)
     abytes = wl.layer_bytes(main_layer.T, shape, n_active)
@@ -591,7 +661,11 @@ def main() -> int:
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": a.workload, "tokens": main_layer.T, "hidden": shape.hidden,
                    "experts": shape.experts, "intermediate": shape.intermediate,
-                   "top_k": shape.top_k, "block_size_m": main_layer.bm, "active_experts": n_active},
+                   "top_k": shape.top_k, "block_size_m": main_layer.bm, "active_experts": n_active,
+                   "weight_layout": a.weight_layout + (
+                       " (FusedMoE(weight_layout='tiled').process_weights_after_loading: the loaded "
+                       "weights re-ordered once; plain_layout = row-major as loaded)"
+                       if a.weight_layout == "tiled" else " (row-major, as loaded)")},
         "layer_tflops": round(tflops, 2), "layer_frac_of_bf16_peak": round(tflops / PEAK_BF16_TFLOPS, 4),
         "layer_algorithmic_gbs": round(gbs, 1),
         "stage_ms": {k: round(v, 4) for k, v in stages.items()},
@@ -602,7 +676,12 @@ def main() -> int:
                      "the headline steps",
         "after_idle": {"ms_per_step": round(ms_after_idle, 4),
                        "tflops": round(flops / (ms_after_idle * 1e-3) / 1e12, 2)},
+        "rotating_weights": {"weight_sets": 4, "ms_per_step": round(ms_rot, 4),
+                             "tflops": round(flops / (ms_rot * 1e-3) / 1e12, 2)},
     }
+    if ms_plain is not None:
+        head["plain_layout"] = {"ms_per_step": round(ms_plain, 4),
+                                "tflops": round(flops / (ms_plain * 1e-3) / 1e12, 2)}
     head.update(out)
     out = head
 

@@ -36,6 +36,11 @@ enum MoeDtype { MOE_F32 = 0, MOE_F16 = 1, MOE_BF16 = 2, MOE_E4M3 = 3 };
    (csrc/dispatch_utils.h:16-24 dispatches the same integral types) */
 enum MoeIdDtype { MOE_ID_I32 = 0, MOE_ID_I64 = 1, MOE_ID_I16 = 2, MOE_ID_I8 = 3, MOE_ID_U8 = 4 };
 enum MoeActivation { MOE_ACT_SILU = 0, MOE_ACT_SWIGLUOAI = 1, MOE_ACT_GELU = 2 };
+/* memory layout of the expert weights handed to moe_fused_experts */
+enum MoeWeightLayout {
+  MOE_WEIGHTS_PLAIN = 0, /* [E, rows, K] row-major, as the reference's loader leaves them       */
+  MOE_WEIGHTS_TILED = 1  /* the same bytes re-ordered once by moe_tile_expert_weights            */
+};
 
 enum MoeError {
   MOE_OK = 0,
@@ -157,8 +162,9 @@ typedef struct MoeFusedExpertsArgs {
   /* tensors */
   const void* x;             /* [T, H] activations, row-major contiguous            */
   void* out;                 /* [T, H] result, same dtype as x                      */
-  const void* w13;           /* [E, 2I, H] gate rows [0,I) then up rows [I,2I)      */
-  const void* w2;            /* [E, H, I]                                           */
+  const void* w13;           /* [E, 2I, H] gate rows [0,I) then up rows [I,2I); or its
+                                tiled form (weight_layout)                          */
+  const void* w2;            /* [E, H, I]; or its tiled form                        */
   const void* w13_bias;      /* [E, 2I] or NULL                                     */
   const void* w2_bias;       /* [E, H] or NULL                                      */
   const float* w13_scale;    /* fp8 only: [E, 2I] per-output-channel scales, else NULL */
@@ -192,6 +198,7 @@ typedef struct MoeFusedExpertsArgs {
      where the library would otherwise enqueue them as one.  Bit 16: the
      workspace already holds the plan (moe_align_block_size_planned). */
   int32_t passes;
+  int32_t weight_layout;     /* MoeWeightLayout of w13 and w2 (both): 0 = plain                   */
   void* stream;
 } MoeFusedExpertsArgs;
 
@@ -226,6 +233,22 @@ int moe_fused_experts_plan_layout(int T, int H, int I, int E, int K, int block_s
  * tokens; plays the role of config["BLOCK_SIZE_M"] chosen by
  * try_get_optimal_moe_config (nanovllm/layers/for_moe/fused_moe.py:354-390). */
 int moe_preferred_block_size(int M, int E, int K, int act_dtype, int weight_dtype);
+
+/* One-time re-ordering of expert weights for the DMA kernels (no counterpart in the reference, whose
+ * loader, nanovllm/layers/fused_moe.py:472-658, leaves `w13_weight [E, 2I, H]` / `w2_weight [E, H, I]`
+ * row-major; the layer owns these tensors, nothing else reads them, so the layer may re-order them
+ * after loading).  `src` [E, rows, K] contiguous -> `dst`, the same number of bytes, as units of 256
+ * weight rows x 128 bytes of K (one unit = what a workgroup stages in LDS per K step), units ordered
+ * [expert][rows / 256][K * elem_bytes / 128]; inside a unit the bytes are in the order they take in
+ * LDS.  `gated` != 0 (w13): a unit holds 128 gate rows and the 128 matching up rows (`interleaved`
+ * != 0: gate row n is source row 2n, up row n is 2n + 1, the swigluoai form).  Every 128-byte piece
+ * of a weight row that the kernels fetch then sits next to the pieces fetched with it: one
+ * sequential 32 KB read per unit instead of 256 pieces a row stride apart.  Results of
+ * moe_fused_experts are bit-identical for both layouts.  rows must be a multiple of 256 and
+ * K * elem_bytes a multiple of 128 (moe_tile_expert_weights_supported returns 1); src != dst. */
+int moe_tile_expert_weights_supported(int rows, int K, int elem_bytes, int gated);
+int moe_tile_expert_weights(const void* src, void* dst, int E, int rows, int K, int elem_bytes, int gated,
+                            int interleaved, void* stream);
 
 /* fp8 helpers (no counterpart in the reference, which asserts the scales are
  * None at nanovllm/layers/for_moe/fused_moe.py:248-249): per-output-channel

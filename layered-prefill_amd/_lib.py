@@ -21,6 +21,7 @@ DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 E4M3_CODE = 3
 ID_DTYPE_CODE = {torch.int32: 0, torch.int64: 1, torch.int16: 2, torch.int8: 3, torch.uint8: 4}
 ACTIVATION_CODE = {"silu": 0, "swigluoai": 1, "gelu": 2}
+WEIGHT_LAYOUT_CODE = {"plain": 0, "tiled": 1}   # MoeWeightLayout
 
 EXPORTS = (
     "moe_last_error", "moe_abi_version", "moe_topk_softmax", "moe_align_workspace_bytes",
@@ -29,6 +30,7 @@ EXPORTS = (
     "moe_quant_rows_e4m3", "moe_gate_topk_softmax", "moe_add_rms_norm",
     "moe_align_can_plan", "moe_align_block_size_planned", "moe_fused_experts_plan_layout",
     "moe_fused_experts_status", "moe_fused_experts_set_wait_limit", "moe_align_block_size_static",
+    "moe_tile_expert_weights", "moe_tile_expert_weights_supported",
 )
 
 
@@ -48,7 +50,7 @@ class MoeFusedExpertsArgs(ctypes.Structure):
         ("weight_dtype", ctypes.c_int32), ("activation", ctypes.c_int32),
         ("apply_router_weight_on_input", ctypes.c_int32),
         ("swiglu_alpha", ctypes.c_float), ("swiglu_limit", ctypes.c_float),
-        ("passes", ctypes.c_int32), ("stream", ctypes.c_void_p),
+        ("passes", ctypes.c_int32), ("weight_layout", ctypes.c_int32), ("stream", ctypes.c_void_p),
     ]
 
 
@@ -103,6 +105,10 @@ def _declare(L: ctypes.CDLL) -> None:
     L.moe_preferred_block_size.argtypes = [i32] * 5
     L.moe_quant_rows_e4m3.restype = i32
     L.moe_quant_rows_e4m3.argtypes = [p, i32, i64, i32, p, p, p]
+    L.moe_tile_expert_weights_supported.restype = i32
+    L.moe_tile_expert_weights_supported.argtypes = [i32] * 4
+    L.moe_tile_expert_weights.restype = i32
+    L.moe_tile_expert_weights.argtypes = [p, p, i32, i32, i32, i32, i32, i32, p]
     L.moe_add_rms_norm.restype = i32
     L.moe_add_rms_norm.argtypes = [p, i64, p, i64, p, i64, p, i32, i64, i32, f32, p]
 

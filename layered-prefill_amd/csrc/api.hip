@@ -36,4 +36,4 @@ int moe_opt_in_lds(MoeLdsOptIn& flags, const void* kernel, int lds_bytes, const 
 
 MOE_EXPORT const char* moe_last_error(void) { return g_last_error; }
 
-MOE_EXPORT int moe_abi_version(void) { return 1; }
+MOE_EXPORT int moe_abi_version(void) { return 2; }

@@ -130,6 +130,11 @@ struct GemmParams {
   int m_major;       // workgroup order inside an XCD: all n-tiles of an m-block are neighbours
   const int32_t* xcd_bounds;  // large-tile kernel: m-block range [b[x], b[x+1]) of XCD x, or null
   int wt_stores;     // large-tile flush: results go out as device-scope write-through stores (one-launch hand-off)
+  // Operands stored as 32 KB units, one per (256 rows, K tile of 128 bytes), each unit the exact
+  // image it has in LDS (row r at r * 128, 16-byte chunk c of the row at chunk c ^ ((r >> 1) & 7)):
+  int w_tiled;       // weights: units [expert][n-tile][K tile] (moe_tile_expert_weights)
+  int a_tiled;       // A operand of the down pass: units [m-block][K tile]
+  int c_tiled;       // result of the gate-up pass written as such units
 };
 
 constexpr int kThreads = 256;
@@ -479,6 +484,7 @@ struct BigCtx {
   int rd_k[4];          // fragment read offsets for the four MFMA steps of a K tile
   int x_row;            // byte offset of this wavefront's first token row in a token unit
   int w_row[4];         // byte offsets of this wavefront's weight fragments in a weight unit
+  int a_step, w_step;   // bytes from one K tile to the next: 128 along a row, 32768 from unit to unit
 };
 
 template <int V>
@@ -584,8 +590,8 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
   // A(kt+2) to fw
   auto next_slot = [](int s) { return s + 2 * kBigUnitBytes >= kBigUnits * kBigUnitBytes ? s + (2 - kBigUnits) * kBigUnitBytes : s + 2 * kBigUnitBytes; };
   int sa = 0, sw = kBigUnitBytes, fa = 3 * kBigUnitBytes, fw = 4 * kBigUnitBytes;
-  const char* a2 = c.a_base + 2 * kBigRowBytes;  // rows of A(kt+2)
-  const char* w1 = c.w_base + kBigRowBytes;      // rows of W(kt+1)
+  const char* a2 = c.a_base + 2 * c.a_step;  // rows of A(kt+2)
+  const char* w1 = c.w_base + c.w_step;      // rows of W(kt+1)
 
   // One K tile.  DO_W: W(kt+1)[4..7] is still to be requested; DO_A: A(kt+2) exists; NEXT:
   // a tile follows; NEXT_W: W(kt+2) exists.
@@ -593,7 +599,7 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
     constexpr bool DO_W = decltype(do_w_tag)::value != 0, DO_A = decltype(do_a_tag)::value != 0;
     constexpr bool NEXT = decltype(next_tag)::value != 0, NEXT_W = decltype(next_w_tag)::value != 0;
     const uint32_t lds_fa = c.dma_lds + fa, lds_fw = c.dma_lds + fw;
-    const char* const w2 = w1 + kBigRowBytes;
+    const char* const w2 = w1 + c.w_step;
     // request q of the tile's first STEPS-1 steps: W(kt+1)[4..7], then A(kt+2)[0..7]
     auto req = [&](auto qt) {
       constexpr int q = decltype(qt)::value;
@@ -626,8 +632,8 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
       constexpr int i = decltype(it)::value;
       if constexpr (NEXT_W) lds_dma16_group<i>(w2, c.w_off[i], lds_w2);
     });
-    a2 += kBigRowBytes;
-    w1 += kBigRowBytes;
+    a2 += c.a_step;
+    w1 += c.w_step;
   };
 
   // fill the ring: W(0) and half of W(1) were requested by the caller as soon as it knew
@@ -635,7 +641,7 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
   static_for<0, 8>([&](auto it) { lds_dma16_group<decltype(it)::value>(c.a_base, c.a_off[decltype(it)::value], c.dma_lds); });
   if (1 < nk) {
     static_for<0, 8>([&](auto it) {
-      lds_dma16_group<decltype(it)::value>(c.a_base + kBigRowBytes, c.a_off[decltype(it)::value], c.dma_lds + 2 * kBigUnitBytes);
+      lds_dma16_group<decltype(it)::value>(c.a_base + c.a_step, c.a_off[decltype(it)::value], c.dma_lds + 2 * kBigUnitBytes);
     });
     wait_vmcnt<kBigDmaPerUnit>();
   } else {
@@ -682,16 +688,16 @@ __device__ __forceinline__ void big_light_mainloop(const BigCtx& c, const char* 
   auto a_slot = [](int k) { return 4 * kBigUnitBytes + (k & 3) * kTokUnit; };
   auto issue_w = [&](int k) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) lds_dma16(c.w_base + k * kBigRowBytes, c.w_off[i], c.dma_lds + w_slot(k) + i * 4096);
+    for (int i = 0; i < 8; ++i) lds_dma16(c.w_base + k * c.w_step, c.w_off[i], c.dma_lds + w_slot(k) + i * 4096);
   };
   auto issue_a = [&](int k) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) lds_dma16(c.a_base + k * kBigRowBytes, c.a_off[i], c.dma_lds + a_slot(k) + i * 4096);
+    for (int i = 0; i < 2; ++i) lds_dma16(c.a_base + k * c.a_step, c.a_off[i], c.dma_lds + a_slot(k) + i * 4096);
   };
   // request order: W(0) W(1) (first half by the caller) A(0) A(1) W(2) A(2), then W(k) A(k) per K tile
   if (1 < nk) {
 #pragma unroll
-    for (int i = 4; i < 8; ++i) lds_dma16(c.w_base + kBigRowBytes, c.w_off[i], c.dma_lds + w_slot(1) + i * 4096);
+    for (int i = 4; i < 8; ++i) lds_dma16(c.w_base + c.w_step, c.w_off[i], c.dma_lds + w_slot(1) + i * 4096);
   }
   issue_a(0);
   if (1 < nk) issue_a(1);
@@ -845,12 +851,23 @@ __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, i
   const int c8 = (lane % LPR) * 8;
   const int ncol = n0 + wn * COLS + c8;
   const bool vec_ok = ncol + 7 < p.N && (p.ldc & 7) == 0;
+  // The gate-up result as 32 KB units of the down pass's A operand: this wavefront's 64 columns
+  // are K tile 2 * (n-tile) + wn of the block, its rows 128 bytes each, chunks in LDS order.
+  // N is a multiple of 64 then, so a wavefront is inside the matrix or has nothing to write.
+  bool tiled = false;
+  if constexpr (GATED) tiled = p.c_tiled != 0;
+  if (tiled && n0 + wn * COLS >= p.N) return;
   // Whole wavefront inside the matrix: no per-lane edge handling.  Real slots come
   // first in a block, so row r is live exactly when r < rows.
-  if (n0 + wn * COLS + COLS <= p.N && (p.ldc & 7) == 0) {
+  if (tiled || (n0 + wn * COLS + COLS <= p.N && (p.ldc & 7) == 0)) {
     const int lrow = lane / LPR;
-    char* const cbase = static_cast<char*>(p.c) + static_cast<int64_t>(ncol) * 2;
-    const int64_t ldc_bytes = static_cast<int64_t>(p.ldc) * 2;
+    char* cbase = static_cast<char*>(p.c) + static_cast<int64_t>(ncol) * 2;
+    int64_t ldc_bytes = static_cast<int64_t>(p.ldc) * 2;
+    if (tiled) {
+      const int64_t unit = static_cast<int64_t>(slot0 >> 8) * (p.N >> 6) + (n0 >> 6) + wn;
+      cbase = static_cast<char*>(p.c) + unit * kBigUnitBytes;
+      ldc_bytes = kBigRowBytes;
+    }
     const char* src = epi + lrow * kEpiRowBytes + c8 * 2;
     for (int r0 = 0; r0 < rows; r0 += RPS * UNR) {
       int crow[UNR];
@@ -859,6 +876,10 @@ __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, i
       for (int u = 0; u < UNR; ++u) {
         const int r = r0 + u * RPS + lrow;  // < 128: rows <= 128 and 128 is a multiple of RPS * UNR
         crow[u] = p.a_by_slot ? s_tok[r] : slot0 + r;
+        if (tiled) {
+          const int rb = (slot0 & 255) + r;  // row inside the block; the row's byte offset carries the chunk
+          crow[u] = rb;
+        }
         gq[u] = *reinterpret_cast<const uint4*>(src + (r0 + u * RPS) * kEpiRowBytes);
         if constexpr (PAIRS) uq[u] = *reinterpret_cast<const uint4*>(src + (r0 + u * RPS) * kEpiRowBytes + 128);
       }
@@ -869,8 +890,10 @@ __device__ __forceinline__ void big_flush(const GemmParams& p, int n0, int wn, i
           out = uint4{gated_pair<El, ACT>(p, gq[u].x, uq[u].x), gated_pair<El, ACT>(p, gq[u].y, uq[u].y),
                       gated_pair<El, ACT>(p, gq[u].z, uq[u].z), gated_pair<El, ACT>(p, gq[u].w, uq[u].w)};
         if (r0 + u * RPS + lrow < rows) {
-          if (p.wt_stores) store16_device_scope(cbase + crow[u] * ldc_bytes, out);
-          else *reinterpret_cast<uint4*>(cbase + crow[u] * ldc_bytes) = out;
+          char* dst = cbase + crow[u] * ldc_bytes;
+          if (tiled) dst += ((lane & 7) ^ ((crow[u] >> 1) & 7)) << 4;
+          if (p.wt_stores) store16_device_scope(dst, out);
+          else *reinterpret_cast<uint4*>(dst) = out;
         }
       }
     }
@@ -983,6 +1006,15 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
   c.a_base = static_cast<const char*>(p.a);
   c.w_base = static_cast<const char*>(p.w) + static_cast<int64_t>(e) * p.w_stride_e * ES;
   c.dma_lds = __builtin_amdgcn_readfirstlane(lds_offset_of(smem) + wave * 1024);
+  c.a_step = c.w_step = kBigRowBytes;
+  if (p.w_tiled) {
+    // unit (n-tile, K tile) of this expert is one 32 KB piece in LDS order: thread tid moves bytes
+    // [16 tid, 16 tid + 16) of each of its eight 4 KB groups
+    c.w_base += static_cast<int64_t>(nt) * nk * kBigUnitBytes;
+    c.w_step = kBigUnitBytes;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) c.w_off[i] = static_cast<uint32_t>(i * 4096 + tid * 16);
+  } else {
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int rr = ld_row + 32 * i;
@@ -998,6 +1030,7 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
     }
     c.w_off[i] = static_cast<uint32_t>(wrow * p.w_stride_n * ES + ld_chunk * 16);
   }
+  }
   // The weights of the first K tile and a half are on their way (ring slots 1 and 3) while
   // the slot ids are still being looked at: they are the cold half of the fill.
   // Neither slot overlaps the side arrays above.
@@ -1006,7 +1039,7 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
   if (1 < nk) {  // the first half of W(1); the main loops request the second
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      lds_dma16(c.w_base + kBigRowBytes, c.w_off[i], c.dma_lds + 3 * kBigUnitBytes + i * 4096);
+      lds_dma16(c.w_base + c.w_step, c.w_off[i], c.dma_lds + 3 * kBigUnitBytes + i * 4096);
   }
   __syncthreads();
   const int nvalid = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
@@ -1032,11 +1065,20 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
     if (p.bias) my_bias = El::ld(static_cast<const typename El::S*>(p.bias)[e * p.bias_stride_e + wr]);
   }
   const int a_groups = (nvalid + 31) >> 5;  // 32-row token groups that hold real slots
+  if (p.a_tiled) {
+    // the block's rows of K tile kt are unit (mb, kt), written in LDS order by the gate-up pass
+    c.a_base += static_cast<int64_t>(mb) * nk * kBigUnitBytes;
+    c.a_step = kBigUnitBytes;
+  }
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     // groups made of padding only re-request group 0 (an L1 hit) so that every
     // token unit is exactly eight loads and the vmcnt bookkeeping stays fixed
     const int gi = i < a_groups ? i : 0;
+    if (p.a_tiled) {
+      c.a_off[i] = static_cast<uint32_t>(gi * 4096 + tid * 16);
+      continue;
+    }
     const int slot = mb * kBigBM + ld_row + 32 * gi;
     int64_t src = slot;
     if (!p.a_by_slot) {
@@ -1409,6 +1451,7 @@ __global__ __launch_bounds__(kThreads, 3) void stream_gemm_kernel(const GemmPara
   // 16 * wave + 8 * j + lane / 8 (j < 2); lane % 8 is the chunk the lane's 16 bytes land in
   const char* a_base = static_cast<const char*>(p.a);
   const char* w_base = static_cast<const char*>(p.w) + static_cast<int64_t>(e) * p.w_stride_e * 2;
+  int w_step = kStRowBytes;  // bytes from one K unit to the next
   uint32_t a_off, w_off[2];
   {
     const int q = lane >> 3;
@@ -1422,6 +1465,20 @@ __global__ __launch_bounds__(kThreads, 3) void stream_gemm_kernel(const GemmPara
     }
     a_off = static_cast<uint32_t>(src * p.lda * 2 + (((lane & 7) ^ ((rr >> 1) & 7)) << 4));
   }
+  if (p.w_tiled) {
+    // Weights in 32 KB units of 256 rows (the large-tile kernel's): this workgroup's rows are one
+    // or two contiguous pieces of every unit of its n-tile, 32 rows apart from a multiple of 32,
+    // so a row's chunks already sit where this kernel's LDS rows want them.
+    constexpr int kBigRows = GATED ? 128 : 256;  // output columns covered by one unit
+    w_base += static_cast<int64_t>(n0 / kBigRows) * (p.Kd / kStBK) * 32768;
+    w_step = 32768;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int rr = 16 * wave + 8 * j + (lane >> 3);
+      const int R = GATED ? ((rr >> 5) * 128 + (n0 % kBigRows) + (rr & 31)) : ((n0 % kBigRows) + rr);
+      w_off[j] = static_cast<uint32_t>(R * kStRowBytes + ((lane & 7) << 4));
+    }
+  } else {
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int rr = 16 * wave + 8 * j + (lane >> 3);
@@ -1437,6 +1494,7 @@ __global__ __launch_bounds__(kThreads, 3) void stream_gemm_kernel(const GemmPara
     }
     w_off[j] = static_cast<uint32_t>(wrow * p.w_stride_n * 2 + (((lane & 7) ^ ((rr >> 1) & 7)) << 4));
   }
+  }
   const uint32_t lds0 = lds_offset_of(smem);
   const uint32_t dma_w = __builtin_amdgcn_readfirstlane(lds0 + 16 * wave * kStRowBytes);
   const uint32_t dma_a = __builtin_amdgcn_readfirstlane(lds0 + kStWBytes + 8 * wave * kStRowBytes);
@@ -1444,7 +1502,7 @@ __global__ __launch_bounds__(kThreads, 3) void stream_gemm_kernel(const GemmPara
     const uint32_t ring = (u % kStUnits) * kStUnitBytes;
     lds_dma16(a_base + u * kStRowBytes, a_off, dma_a + ring);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) lds_dma16(w_base + u * kStRowBytes, w_off[j], dma_w + ring + j * 1024);
+    for (int j = 0; j < 2; ++j) lds_dma16(w_base + static_cast<int64_t>(u) * w_step, w_off[j], dma_w + ring + j * 1024);
   };
 
   f32x16 acc0, acc1;
@@ -1620,6 +1678,9 @@ int launch_bm(GemmParams& p, int block_size, int64_t sorted_cap, hipStream_t s) 
     if (block_size == kStBM && p.Kd % kStBK == 0 && offsets_fit)
       return launch_stream<Mma, GATED>(p, sorted_cap, s);
   }
+  if (p.w_tiled)
+    return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: tiled weights run on the large-tile kernel (block_size a multiple "
+                    "of 256) and the streaming kernel (block_size 32) only, not with block_size %d", block_size);
   if (block_size % 128 == 0) {
     p.num_m_blocks = static_cast<int>((sorted_cap + 127) / 128);
     p.num_n_tiles = (p.N + (GATED ? 64 : 128) - 1) / (GATED ? 64 : 128);
@@ -1640,7 +1701,61 @@ int launch_bm(GemmParams& p, int block_size, int64_t sorted_cap, hipStream_t s) 
 
 int elem_size(int dtype) { return dtype == MOE_F32 ? 4 : (dtype == MOE_E4M3 ? 1 : 2); }
 
+// Copies expert weights [E, rows, K] into the unit layout the DMA kernels fetch with plain
+// sequential requests.  One workgroup per unit (expert e, n-tile nt, K tile kt): 256 weight rows of
+// 128 bytes.  Gated matrices (w13): unit rows [0, 128) are gate rows 128 nt .. + 127, unit rows
+// [128, 256) the matching up rows (rows 2n and 2n + 1 when gate and up are interleaved); others
+// (w2): rows 256 nt .. + 255.  Inside a unit row r sits at r * 128 and its 16-byte chunk c at chunk
+// c ^ ((r >> 1) & 7), the place it has in LDS.
+__global__ __launch_bounds__(kThreads) void tile_weights_kernel(const char* __restrict__ src, char* __restrict__ dst,
+                                                                int rows, int64_t row_bytes, int n_tiles, int k_tiles,
+                                                                int gated, int interleaved) {
+  const int64_t unit = blockIdx.x;
+  const int kt = static_cast<int>(unit % k_tiles);
+  const int nt = static_cast<int>((unit / k_tiles) % n_tiles);
+  const int64_t e = unit / k_tiles / n_tiles;
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int r = (tid >> 3) + 32 * i, pos = tid & 7;
+    const int chunk = pos ^ ((r >> 1) & 7);
+    int64_t srow;
+    if (gated) {
+      const int half = r >> 7, n = nt * 128 + (r & 127);
+      srow = interleaved ? 2 * n + half : static_cast<int64_t>(half) * (rows / 2) + n;
+    } else {
+      srow = static_cast<int64_t>(nt) * 256 + r;
+    }
+    const uint4 v = *reinterpret_cast<const uint4*>(src + (e * rows + srow) * row_bytes + kt * 128 + chunk * 16);
+    *reinterpret_cast<uint4*>(dst + unit * kBigUnitBytes + r * 128 + pos * 16) = v;
+  }
+}
+
 }  // namespace
+
+MOE_EXPORT int moe_tile_expert_weights_supported(int rows, int K, int elem_bytes, int gated) {
+  if (rows < 1 || K < 1 || (elem_bytes != 1 && elem_bytes != 2)) return 0;
+  return rows % 256 == 0 && (static_cast<int64_t>(K) * elem_bytes) % 128 == 0 ? 1 : 0;
+}
+
+MOE_EXPORT int moe_tile_expert_weights(const void* src, void* dst, int E, int rows, int K, int elem_bytes, int gated,
+                                       int interleaved, void* stream) {
+  if (!src || !dst || E < 1) return moe_fail(MOE_ERR_ARG, "tile_expert_weights: null pointer or E=%d", E);
+  if (!moe_tile_expert_weights_supported(rows, K, elem_bytes, gated))
+    return moe_fail(MOE_ERR_UNSUPPORTED, "tile_expert_weights: rows=%d must be a multiple of 256 and K=%d x %d bytes a "
+                    "multiple of 128", rows, K, elem_bytes);
+  if (src == dst) return moe_fail(MOE_ERR_ARG, "tile_expert_weights: source and destination must differ");
+  if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15u)
+    return moe_fail(MOE_ERR_ARG, "tile_expert_weights: buffers must be 16-byte aligned");
+  const int64_t row_bytes = static_cast<int64_t>(K) * elem_bytes;
+  const int n_tiles = rows / 256, k_tiles = static_cast<int>(row_bytes / 128);
+  const int64_t units = static_cast<int64_t>(E) * n_tiles * k_tiles;
+  if (units > INT32_MAX) return moe_fail(MOE_ERR_ARG, "tile_expert_weights: %lld units", static_cast<long long>(units));
+  hipLaunchKernelGGL(tile_weights_kernel, dim3(static_cast<unsigned>(units)), dim3(kThreads), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const char*>(src), static_cast<char*>(dst), rows,
+                     row_bytes, n_tiles, k_tiles, gated ? 1 : 0, interleaved ? 1 : 0);
+  return moe_check_launch("tile_expert_weights");
+}
 
 MOE_EXPORT int moe_preferred_block_size(int M, int E, int K, int act_dtype, int weight_dtype) {
   if (E < 1) return 64;
@@ -1731,6 +1846,21 @@ static int check_fused_args(const MoeFusedExpertsArgs* a, int64_t* cap, int64_t*
   if ((reinterpret_cast<uintptr_t>(a->x) | reinterpret_cast<uintptr_t>(a->w13) |
        reinterpret_cast<uintptr_t>(a->w2) | reinterpret_cast<uintptr_t>(a->out)) & 15u)
     return moe_fail(MOE_ERR_ARG, "fused_experts: tensors must be 16-byte aligned");
+  if (a->weight_layout != MOE_WEIGHTS_PLAIN && a->weight_layout != MOE_WEIGHTS_TILED)
+    return moe_fail(MOE_ERR_ARG, "fused_experts: unknown weight_layout %d", a->weight_layout);
+  if (a->weight_layout == MOE_WEIGHTS_TILED) {
+    if (fp8 || a->act_dtype == MOE_F32)
+      return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: tiled weights are for bf16 and fp16 only");
+    if (!moe_tile_expert_weights_supported(2 * a->I, a->H, 2, 1) || !moe_tile_expert_weights_supported(a->H, a->I, 2, 0))
+      return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: tiled weights need I a multiple of 128 and H a multiple of 256 "
+                      "(I=%d, H=%d)", a->I, a->H);
+    if (a->w13_stride_n != a->H || a->w13_stride_e != 2LL * a->I * a->H || a->w2_stride_n != a->I ||
+        a->w2_stride_e != static_cast<int64_t>(a->H) * a->I)
+      return moe_fail(MOE_ERR_ARG, "fused_experts: tiled weights are contiguous [E, rows, K] buffers");
+    if (a->block_size % kBigBM != 0 && a->block_size != kStBM)
+      return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: tiled weights need block_size 32 or a multiple of 256, not %d",
+                      a->block_size);
+  }
   const int64_t numel = static_cast<int64_t>(a->T) * a->K;
   const int64_t need_cap = numel + static_cast<int64_t>(a->E) * (a->block_size - 1);
   if (a->sorted_cap < need_cap)
@@ -1747,18 +1877,25 @@ static int check_fused_args(const MoeFusedExpertsArgs* a, int64_t* cap, int64_t*
   return MOE_OK;
 }
 
-// Whether this call enqueues the two GEMM passes as one launch (16-bit dtypes, blocks that are
-// multiples of 256 slots, both passes requested, operands within the DMA kernels' 32-bit offsets).
-static bool uses_one_launch(const MoeFusedExpertsArgs* a, int64_t cap) {
+// Whether both GEMM passes of this call run on the 16-bit large-tile kernel, which then keeps the
+// intermediate as 32 KB units in the workspace (I a multiple of 64 is part of big_16bit_ok).
+static bool inter_units_ok(const MoeFusedExpertsArgs* a, int64_t cap) {
   if (a->block_size % kBigBM != 0 || a->act_dtype == MOE_F32 || a->weight_dtype == MOE_E4M3) return false;
-  const int passes = (a->passes & 7) ? a->passes : (a->passes | 7);
-  if ((passes & 3) != 3 || (passes & 8)) return false;
   GemmParams p1{}, p2{};
   p1.numel = p2.numel = static_cast<int>(static_cast<int64_t>(a->T) * a->K);
   p1.top_k = p2.top_k = a->K;
   p1.lda = a->H; p1.Kd = a->H; p1.N = a->I; p1.w_stride_n = a->w13_stride_n; p1.a_by_slot = 0;
   p2.lda = a->I; p2.Kd = a->I; p2.N = a->H; p2.w_stride_n = a->w2_stride_n; p2.a_by_slot = 1;
   return big_16bit_ok(p1, true, a->block_size, cap) && big_16bit_ok(p2, false, a->block_size, cap);
+}
+
+// Whether this call enqueues the two GEMM passes as one launch (16-bit dtypes, blocks that are
+// multiples of 256 slots, both passes requested, operands within the DMA kernels' 32-bit offsets).
+static bool uses_one_launch(const MoeFusedExpertsArgs* a, int64_t cap) {
+  if (a->block_size % kBigBM != 0 || a->act_dtype == MOE_F32 || a->weight_dtype == MOE_E4M3) return false;
+  const int passes = (a->passes & 7) ? a->passes : (a->passes | 7);
+  if ((passes & 3) != 3 || (passes & 8)) return false;
+  return inter_units_ok(a, cap);
 }
 
 MOE_EXPORT int moe_fused_experts_set_wait_limit(int polls) {
@@ -1811,6 +1948,7 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.limit = a->swiglu_limit;
   p.activation = a->activation;
   p.interleaved = a->activation == MOE_ACT_SWIGLUOAI;
+  p.w_tiled = a->weight_layout == MOE_WEIGHTS_TILED ? 1 : 0;
   const int32_t* plan_bounds = nullptr;
   int32_t* plan_done = nullptr;
   if (a->block_size % kBigBM == 0 && a->act_dtype != MOE_F32) {
@@ -1834,6 +1972,12 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.mul_weight = a->apply_router_weight_on_input ? 1 : 0;
   const int passes = (a->passes & 7) ? a->passes : (a->passes | 7);
   int rc = MOE_OK;
+  // When both passes run on the 16-bit large-tile kernel the intermediate lives in the workspace as
+  // 32 KB units (256 slots x one K tile of the down pass, LDS order): the gate-up flush writes whole
+  // units and the down pass fetches each with plain sequential requests.  The choice depends on the
+  // sizes only, never on `passes`, so single passes enqueued apart agree on it.
+  const bool inter_tiled = plan_bounds && !fp8 && inter_units_ok(a, cap);
+  p.c_tiled = inter_tiled ? 1 : 0;
   if (plan_bounds && !fp8 && (passes & 3) == 3 && !(passes & 8)) {
     // 16-bit dtypes on the large-tile kernel: both passes in one launch
     GemmParams p2 = p;
@@ -1841,6 +1985,7 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
     p2.bias = a->w2_bias; p2.bias_stride_e = a->H;
     p2.c = c3; p2.ldc = a->H; p2.Kd = a->I; p2.N = a->H; p2.a_by_slot = 1;
     p2.mul_weight = a->apply_router_weight_on_input ? 0 : 1;
+    p2.c_tiled = 0; p2.a_tiled = inter_tiled ? 1 : 0;
     if (big_16bit_ok(p, true, a->block_size, cap) && big_16bit_ok(p2, false, a->block_size, cap)) {
       int32_t* status = const_cast<int32_t*>(plan_bounds) + kBigStatusWord;
       rc = a->act_dtype == MOE_BF16 ? launch_big_fused<MmaBF16>(p, p2, a->block_size, cap, plan_done, status, s)
@@ -1870,6 +2015,7 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.c = c3; p.ldc = a->H; p.Kd = a->I; p.N = a->H; p.a_by_slot = 1;
   p.mul_weight = a->apply_router_weight_on_input ? 0 : 1;
   p.xcd_bounds = plan_bounds;
+  p.c_tiled = 0; p.a_tiled = inter_tiled ? 1 : 0;
   if (fp8 && (passes & 2)) {
     // the activated intermediate is quantised per slot row the same way
     rc = moe_quant_slot_rows_e4m3(inter, a->act_dtype, rows, a->I, reinterpret_cast<uint8_t*>(iq), is,

@@ -140,18 +140,20 @@ def fused_experts(hidden_states: torch.Tensor,
                   a1_scale: Optional[torch.Tensor] = None,
                   a2_scale: Optional[torch.Tensor] = None,
                   block_shape: Optional[list] = None,
-                  allow_deep_gemm: bool = False) -> torch.Tensor:
-    """nanovllm/layers/for_moe/fused_moe.py:422-460."""
+                  allow_deep_gemm: bool = False,
+                  weight_layout: str = "plain") -> torch.Tensor:
+    """nanovllm/layers/for_moe/fused_moe.py:422-460.  ``weight_layout`` (not in the
+    reference) is "tiled" when ``w1`` and ``w2`` came out of ``ops.tile_expert_weights``."""
     if inplace:
         fused_experts_impl(hidden_states, w1, w2, topk_weights, topk_ids, True, activation,
                            apply_router_weight_on_input, per_channel_quant, global_num_experts,
                            expert_map, w1_scale, w2_scale, w1_zp, w2_zp, a1_scale, a2_scale,
-                           block_shape, w1_bias, w2_bias)
+                           block_shape, w1_bias, w2_bias, weight_layout)
         return hidden_states
     return fused_experts_impl(hidden_states, w1, w2, topk_weights, topk_ids, False, activation,
                               apply_router_weight_on_input, per_channel_quant, global_num_experts,
                               expert_map, w1_scale, w2_scale, w1_zp, w2_zp, a1_scale, a2_scale,
-                              block_shape, w1_bias, w2_bias)
+                              block_shape, w1_bias, w2_bias, weight_layout)
 
 
 def fused_experts_workspace_bytes(tokens: int, hidden: int, intermediate: int, experts: int,
@@ -171,7 +173,8 @@ def launch_fused_experts(x: torch.Tensor, out: torch.Tensor, w1: torch.Tensor, w
                          block_size: int, activation: str = "silu",
                          apply_router_weight_on_input: bool = False,
                          weight_code: Optional[int] = None,
-                         workspace: Optional[torch.Tensor] = None, passes: int = 0) -> MoeFusedExpertsArgs:
+                         workspace: Optional[torch.Tensor] = None, passes: int = 0,
+                         weight_layout: str = "plain") -> MoeFusedExpertsArgs:
     """One call of the C entry point ``moe_fused_experts`` on already aligned
     tokens (the part of nanovllm/layers/for_moe/fused_moe.py:579-631 after
     moe_align_block_size).  ``workspace`` (uint8) is allocated when not given;
@@ -208,7 +211,8 @@ def launch_fused_experts(x: torch.Tensor, out: torch.Tensor, w1: torch.Tensor, w
         sorted_cap=sorted_token_ids.numel(), act_dtype=act_code, weight_dtype=weight_code,
         activation=_lib.ACTIVATION_CODE[activation],
         apply_router_weight_on_input=int(apply_router_weight_on_input),
-        swiglu_alpha=1.702, swiglu_limit=7.0, passes=passes, stream=stream_ptr(x.device))
+        swiglu_alpha=1.702, swiglu_limit=7.0, passes=passes,
+        weight_layout=_lib.WEIGHT_LAYOUT_CODE[weight_layout], stream=stream_ptr(x.device))
     with torch.cuda.device(x.device):
         check(L.moe_fused_experts(args))
     args._keepalive = (workspace,)
@@ -262,7 +266,8 @@ def fused_experts_impl(hidden_states: torch.Tensor,
                        a2_scale: Optional[torch.Tensor] = None,
                        block_shape: Optional[list] = None,
                        w1_bias: Optional[torch.Tensor] = None,
-                       w2_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                       w2_bias: Optional[torch.Tensor] = None,
+                       weight_layout: str = "plain") -> torch.Tensor:
     """nanovllm/layers/for_moe/fused_moe.py:461-633: align -> gate-up GEMM with
     the gated activation -> down GEMM times the routed weight -> top-k sum, in
     chunks of 64K tokens."""
@@ -279,6 +284,8 @@ def fused_experts_impl(hidden_states: torch.Tensor,
     assert w1_zp is None and w2_zp is None and block_shape is None and expert_map is None
     if activation not in _lib.ACTIVATION_CODE:
         raise ValueError(f"Unsupported FusedMoe activation: {activation}")
+    if weight_layout not in _lib.WEIGHT_LAYOUT_CODE:
+        raise ValueError(f"Unsupported weight_layout: {weight_layout}")
 
     fp8 = w1.dtype in _FP8_DTYPES or (w1_scale is not None)
     if fp8:
@@ -360,7 +367,8 @@ def fused_experts_impl(hidden_states: torch.Tensor,
                                     w1_bias, w2_bias, w1_scale, w2_scale, curr_w, sorted_token_ids,
                                     expert_ids, num_tokens_post_padded, bm, activation,
                                     apply_router_weight_on_input, weight_code=weight_code,
-                                    workspace=workspace, passes=16 if plan is not None else 0)
+                                    workspace=workspace, passes=16 if plan is not None else 0,
+                                    weight_layout=weight_layout)
         if _CHECK_HANDOFF and not torch.cuda.is_current_stream_capturing():  # the check waits for the stream
             fused_experts_status(args)
     return out_hidden_states

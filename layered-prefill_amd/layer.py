@@ -104,7 +104,29 @@ class UnquantizedFusedMoEMethod:
             w2_bias=layer.w2_bias if hasattr(layer, "w2_bias") else None,
             topk_weights=topk_weights, topk_ids=topk_ids, inplace=True, activation=activation,
             apply_router_weight_on_input=apply_router_weight_on_input,
-            global_num_experts=global_num_experts, expert_map=expert_map)
+            global_num_experts=global_num_experts, expert_map=expert_map,
+            weight_layout="tiled" if getattr(layer, "weights_tiled", False) else "plain")
+
+    def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
+        """With ``FusedMoE(weight_layout="tiled")``: re-orders ``w13_weight`` and ``w2_weight`` once,
+        after the checkpoint is in, into the unit order the DMA kernels fetch sequentially
+        (``ops.tile_expert_weights``).  The parameters keep their shape and dtype but no longer
+        hold weight [e, r, k] at [e, r, k]; ``layer.weights_tiled`` records it and ``apply`` hands
+        it on.  The reference has no such step: its loader
+        (nanovllm/layers/fused_moe.py:472-658) leaves the tensors row-major and only this layer
+        reads them.  Shapes the tiling does not take (I not a multiple of 128, H not a multiple
+        of 256, fp32) stay row-major."""
+        from . import ops
+        if getattr(layer, "weight_layout", "plain") != "tiled" or getattr(layer, "weights_tiled", False):
+            return
+        w13, w2 = layer.w13_weight.data, layer.w2_weight.data
+        if not (w13.is_cuda and ops.tile_expert_weights_supported(w13, True)
+                and ops.tile_expert_weights_supported(w2, False)):
+            return
+        interleaved = layer.activation == "swigluoai"
+        layer.w13_weight.data = ops.tile_expert_weights(w13, True, interleaved)
+        layer.w2_weight.data = ops.tile_expert_weights(w2, False)
+        layer.weights_tiled = True
 
 
 class Fp8E4M3FusedMoEMethod(UnquantizedFusedMoEMethod):
@@ -159,7 +181,7 @@ class FusedMoE(torch.nn.Module):
                  e_score_correction_bias: Optional[torch.Tensor] = None,
                  apply_router_weight_on_input: bool = False, activation: str = "silu",
                  num_redundant_experts: int = 0, has_bias: bool = False,
-                 quantization: Optional[str] = None):
+                 quantization: Optional[str] = None, weight_layout: str = "plain"):
         super().__init__()
         if params_dtype is None:
             params_dtype = torch.get_default_dtype()
@@ -187,6 +209,12 @@ class FusedMoE(torch.nn.Module):
         self.e_score_correction_bias = e_score_correction_bias
         self.apply_router_weight_on_input = apply_router_weight_on_input
         self.activation = activation
+        # `weight_layout` has no counterpart in the reference constructor: "tiled" makes
+        # process_weights_after_loading re-order the expert weights for the DMA kernels
+        if weight_layout not in ("plain", "tiled"):
+            raise ValueError(f"unsupported weight_layout {weight_layout!r}")
+        self.weight_layout = weight_layout
+        self.weights_tiled = False
         if self.scoring_func != "softmax" and not self.use_grouped_topk:
             raise ValueError("Only softmax scoring function is supported for non-grouped topk.")
         self.moe_config = MoEConfig(

@@ -247,6 +247,31 @@ def add_rms_norm(out: torch.Tensor, residual: torch.Tensor, x: torch.Tensor, wei
     _norm_call(out, residual, x, weight, eps, "add_rms_norm")
 
 
+def tile_expert_weights_supported(w: torch.Tensor, gated: bool) -> bool:
+    """Whether ``tile_expert_weights`` takes this [E, rows, K] tensor: bf16 / fp16, contiguous, rows
+    a multiple of 256 (gate and up halves of 128 each when gated), K a multiple of 64."""
+    return bool(w.dim() == 3 and w.dtype in (torch.bfloat16, torch.float16) and w.is_contiguous()
+                and lib().moe_tile_expert_weights_supported(w.size(1), w.size(2), w.element_size(), int(gated)))
+
+
+def tile_expert_weights(w: torch.Tensor, gated: bool, interleaved: bool = False) -> torch.Tensor:
+    """[E, rows, K] expert weights -> a new tensor of the same shape and dtype whose bytes are in the
+    unit order of ``moe_tile_expert_weights`` (units of 256 rows x 128 bytes of K in the order they
+    take in LDS; for ``gated`` w13, 128 gate rows with their 128 up rows).  To be handed to
+    ``fused_experts`` with ``weight_layout="tiled"``; element [e, r, k] of the result is *not*
+    weight [e, r, k].  No counterpart in the reference (its loader leaves the tensors row-major,
+    nanovllm/layers/fused_moe.py:472-658)."""
+    require_gpu_tensor(w, "w")
+    if not tile_expert_weights_supported(w, gated):
+        raise RuntimeError(f"tile_expert_weights: {tuple(w.shape)} {w.dtype} is not tileable: contiguous bf16/fp16 "
+                           "[E, rows, K] with rows % 256 == 0 and K % 64 == 0 expected")
+    out = torch.empty_like(w)
+    with torch.cuda.device(w.device):
+        check(lib().moe_tile_expert_weights(w.data_ptr(), out.data_ptr(), w.size(0), w.size(1), w.size(2),
+                                            w.element_size(), int(gated), int(interleaved), stream_ptr(w.device)))
+    return out
+
+
 def quant_rows_e4m3(w: torch.Tensor):
     """[..., cols] -> (e4m3fn codes as uint8 of the same shape, fp32 scales [...]):
     per-row s = amax|w| / 448.  No counterpart in the reference."""

@@ -661,3 +661,96 @@ def test_longer_sorted_ids_buffer_is_accepted_and_its_surplus_ignored(moe, oracl
         torch.cuda.synchronize()
         assert torch.equal(out, exact)
         _close(out, oracle.fused_experts_ref(x.cpu(), w13.cpu(), w2.cpu(), tw.cpu(), ids.cpu()))
+
+
+def _tile_reference(w: torch.Tensor, gated: bool, interleaved: bool) -> torch.Tensor:
+    """The unit order of ``moe_tile_expert_weights`` written out with index arithmetic on
+    the CPU: units [expert][rows / 256][K / 64] of 256 rows x 8 chunks of 8 elements; unit
+    row r holds source row (gated: gate row 128 nt + r for r < 128, its up row for r >= 128;
+    else row 256 nt + r) and its chunk c sits at position c ^ ((r >> 1) & 7)."""
+    E, rows, K = w.shape
+    n_tiles, k_tiles = rows // 256, K // 64
+    r = torch.arange(256)
+    nt = torch.arange(n_tiles).view(-1, 1)
+    if gated:
+        half, n = r // 128, nt * 128 + (r % 128)
+        srow = 2 * n + half if interleaved else half * (rows // 2) + n
+    else:
+        srow = nt * 256 + r
+    pos = torch.arange(8)
+    chunk = pos.view(1, 8) ^ ((r.view(256, 1) >> 1) & 7)                      # [256, 8]
+    src = w.view(E, rows, k_tiles, 8, 8)                                       # [E, row, kt, chunk, 8]
+    out = torch.empty(E, n_tiles, k_tiles, 256, 8, 8, dtype=w.dtype)
+    for t in range(n_tiles):
+        rows_t = src[:, srow[t]]                                               # [E, 256, kt, chunk, 8]
+        picked = rows_t[:, r.view(256, 1), :, chunk]                           # [256, 8, E, kt, 8]
+        out[:, t] = picked.permute(2, 3, 0, 1, 4)
+    return out.reshape(E, rows, K)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("gated,interleaved", [(True, False), (True, True), (False, False)])
+def test_tile_expert_weights_is_the_documented_unit_order(moe, dev, dtype, gated, interleaved):
+    g = torch.Generator().manual_seed(3)
+    w = torch.randn(3, 512, 192, generator=g).to(dtype)
+    got = moe.ops.tile_expert_weights(w.to(dev), gated, interleaved)
+    torch.cuda.synchronize()
+    assert got.shape == w.shape and got.dtype == w.dtype
+    assert torch.equal(got.cpu().view(torch.int16), _tile_reference(w, gated, interleaved).view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,K", [(40, 2), (700, 4), (3000, 2)])
+@pytest.mark.parametrize("activation,bias", [("silu", False), ("swigluoai", True), ("gelu", False)])
+def test_tiled_weights_give_bit_identical_results(moe, oracle, dev, dtype, T, K, activation, bias):
+    """Streaming kernel (40 tokens: blocks of 32) and large-tile kernel (blocks of 256, one
+    launch for both passes) on weights re-ordered by ``tile_expert_weights``: the same bits
+    as on the row-major weights, and within tolerance of the fp32 oracle."""
+    E, H, I = 8, 512, 256
+    print(f"tiled weights {dtype} T={T} K={K} {activation} bias={bias}", flush=True)
+    x, w13, w2, logits = _layer(E, H, I, T, K, 31 + T, dtype, wstd=0.02)  # the benchmark's weight scale
+    g = torch.Generator().manual_seed(5)
+    b13 = (torch.randn(E, 2 * I, generator=g) * 0.1).to(dtype) if bias else None
+    b2 = (torch.randn(E, H, generator=g) * 0.1).to(dtype) if bias else None
+    tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
+    dv = lambda t: None if t is None else t.to(dev)
+    w13d, w2d = w13.to(dev), w2.to(dev)
+    plain = moe.fused_experts(x.to(dev), w13d, w2d, dv(b13), dv(b2), tw.to(dev), ids.to(dev), activation=activation)
+    w13t = moe.ops.tile_expert_weights(w13d, True, activation == "swigluoai")
+    w2t = moe.ops.tile_expert_weights(w2d, False)
+    tiled = moe.fused_experts(x.to(dev), w13t, w2t, dv(b13), dv(b2), tw.to(dev), ids.to(dev), activation=activation,
+                              weight_layout="tiled")
+    torch.cuda.synchronize()
+    assert torch.equal(plain.view(torch.int16), tiled.view(torch.int16))
+    _close(tiled, oracle.fused_experts_ref(x, w13, w2, tw, ids, activation=activation, w1_bias=b13, w2_bias=b2))
+
+
+def test_tiled_weights_are_rejected_where_no_kernel_reads_them(moe, oracle, dev, monkeypatch):
+    x, w13, w2, logits = _layer(8, 512, 256, 300, 2, 2, torch.bfloat16)
+    tw, ids, _ = oracle.topk_softmax(logits, 2, renormalize=True)
+    w13t = moe.ops.tile_expert_weights(w13.to(dev), True)
+    w2t = moe.ops.tile_expert_weights(w2.to(dev), False)
+    monkeypatch.setattr(moe.fused_moe, "try_get_optimal_moe_config", lambda *a, **k: {"BLOCK_SIZE_M": 64})
+    with pytest.raises(RuntimeError, match="tiled weights"):
+        moe.fused_experts(x.to(dev), w13t, w2t, None, None, tw.to(dev), ids.to(dev), weight_layout="tiled")
+    with pytest.raises(RuntimeError, match="not tileable"):
+        moe.ops.tile_expert_weights(torch.zeros(2, 200, 64, dtype=torch.bfloat16, device=dev), True)
+
+
+def test_fused_moe_layer_with_tiled_weights(moe, oracle, dev):
+    """``FusedMoE(weight_layout="tiled")``: process_weights_after_loading re-orders the loaded
+    parameters once; the forward result equals the row-major layer's bit for bit."""
+    E, H, I, T, K = 8, 256, 128, 500, 2
+    x, w13, w2, logits = _layer(E, H, I, T, K, 77, torch.bfloat16)
+    outs = []
+    for layout in ("plain", "tiled"):
+        layer = moe.FusedMoE(E, K, H, I, params_dtype=torch.bfloat16, weight_layout=layout).to(dev)
+        layer.w13_weight.data.copy_(w13)
+        layer.w2_weight.data.copy_(w2)
+        layer.process_weights_after_loading()
+        assert layer.weights_tiled == (layout == "tiled")
+        outs.append(layer(x.to(dev).clone(), logits.to(dev)))
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+    tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
+    _close(outs[1], oracle.fused_experts_ref(x, w13, w2, tw, ids))

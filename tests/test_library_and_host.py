@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol(moe):
     for name in _declared_functions():
         assert hasattr(lib, name), f"{name} declared in include/moe_gfx950.h but not exported"
     assert set(_declared_functions()) == set(moe._lib.EXPORTS)
-    assert moe._lib.lib().moe_abi_version() == 1
+    assert moe._lib.lib().moe_abi_version() == 2
 
 
 def test_struct_layout_matches_header(moe):
@@ -96,10 +96,12 @@ def test_signatures_match_the_reference_interface(moe):
     assert list(inspect.signature(moe.moe_align_block_size).parameters) == ["topk_ids", "block_size", "num_experts"]
     assert list(inspect.signature(moe.fused_topk).parameters) == ["hidden_states", "gating_output", "topk", "renormalize"]
     fe = inspect.signature(moe.fused_experts).parameters
-    assert list(fe) == ["hidden_states", "w1", "w2", "w1_bias", "w2_bias", "topk_weights", "topk_ids", "inplace",
-                        "activation", "apply_router_weight_on_input", "per_channel_quant", "global_num_experts",
-                        "expert_map", "w1_scale", "w2_scale", "w1_zp", "w2_zp", "a1_scale", "a2_scale",
-                        "block_shape", "allow_deep_gemm"]
+    # the reference's parameters, in its order; what this build adds comes after them, with a default
+    assert list(fe)[:21] == ["hidden_states", "w1", "w2", "w1_bias", "w2_bias", "topk_weights", "topk_ids", "inplace",
+                             "activation", "apply_router_weight_on_input", "per_channel_quant", "global_num_experts",
+                             "expert_map", "w1_scale", "w2_scale", "w1_zp", "w2_zp", "a1_scale", "a2_scale",
+                             "block_shape", "allow_deep_gemm"]
+    assert list(fe)[21:] == ["weight_layout"] and fe["weight_layout"].default == "plain"
     assert fe["inplace"].default is False and fe["activation"].default == "silu"
     # csrc/ops.cpp:29-31,46-60
     assert list(inspect.signature(moe.ops.topk_softmax).parameters)[:4] == [
