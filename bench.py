@@ -120,9 +120,10 @@ class Layer:
         return other
 
     def step(self):
-        moe, s = self.moe, self.shape
-        tw, ids, _ = moe.fused_topk(self.x, self.logits, s.top_k, True)
-        return self.experts(self.x, tw, ids)
+        """The layer call as ``FusedMoE.forward`` makes it (``UnquantizedFusedMoEMethod.apply``):
+        ``fused_topk`` then ``fused_experts`` through ``fused_topk_experts``."""
+        return self.moe.fused_topk_experts(self.x, self.logits, self.w13_run, self.w2_run, self.shape.top_k, True,
+                                           weight_layout=self.layout)
 
     def step_instrumented(self, ev):
         """Same work with an event after every stage (5 stages -> 6 events), the two
@@ -173,9 +174,8 @@ def time_steps_rotating(layer: Layer, steps: int, warmup: int, nsets: int = 4):
     moe, s = layer.moe, layer.shape
 
     def step(i):
-        tw, ids, _ = moe.fused_topk(layer.x, layer.logits, s.top_k, True)
         w13, w2 = sets[i % nsets]
-        return moe.fused_experts(layer.x, w13, w2, None, None, tw, ids, weight_layout=layer.layout)
+        return moe.fused_topk_experts(layer.x, layer.logits, w13, w2, s.top_k, True, weight_layout=layer.layout)
 
     for i in range(warmup):
         step(i)
@@ -307,8 +307,8 @@ def trace_mix(moe, layer: Layer, steps: int):
         x, logits = x.to(layer.dev), logits.to(layer.dev)
 
         def step():
-            tw, ids, _ = moe.fused_topk(x, logits, s.top_k, True)
-            return layer.experts(x, tw, ids)
+            return moe.fused_topk_experts(x, logits, layer.w13_run, layer.w2_run, s.top_k, True,
+                                          weight_layout=layer.layout)
 
         # sustained rate per bucket: about 40 ms of warm-up, then `steps` timed calls
         for _ in range(max(3, min(200, int(40.0 / (0.1 + b * 1e-4))))):

@@ -130,6 +130,22 @@ int moe_align_block_size_planned(const void* topk_ids, int ids_dtype, int64_t nu
                                  int32_t* plan_done, int plan_num_done, int plan_cap_mb);
 
 
+/* moe_topk_softmax followed by moe_align_block_size (with the plan of
+ * moe_align_block_size_planned when `plan_bounds` is not NULL) as ONE launch, for the small
+ * batches of a decode loop: the reference enqueues these as two ops back to back
+ * (nanovllm/layers/fused_moe.py:693-741 then nanovllm/layers/for_moe/fused_moe.py:575-577), each a
+ * few microseconds, so every launch saved counts.  Results are those of the two calls, bit for bit:
+ * `topk_ids` ([T, K] int32) is what gets aligned.  Served sizes (moe_route_align_supported returns
+ * 1): T <= 512, E a power of two <= 256, K <= E, T * K <= 16384; otherwise MOE_ERR_UNSUPPORTED and
+ * the caller routes and aligns apart.  No workspace. */
+int moe_route_align_supported(int T, int E, int K);
+int moe_route_align_block_size(const float* gating_output, float* topk_weights, int32_t* topk_ids,
+                               int32_t* token_expert_indices, int T, int E, int K, int renormalize,
+                               int block_size, int32_t* sorted_token_ids, int64_t sorted_cap,
+                               int32_t* expert_ids, int64_t expert_cap, int32_t* num_tokens_post_pad,
+                               void* stream, int32_t* plan_bounds, int32_t* plan_done, int plan_num_done,
+                               int plan_cap_mb);
+
 /* Replaces `silu_and_mul` (csrc/activation_kernels.cu:68-87, bound at
  * csrc/ops.cpp:29-31,99-103): out[r,i] = T(silu(in[r,i])) * in[r,d+i]. */
 int moe_silu_and_mul(void* out, const void* in, int64_t rows, int d, int dtype, void* stream);

@@ -13,7 +13,7 @@ CPU or PyTorch fallback.
 """
 from . import _lib, ops, fused_moe, layer, loader, schedule, workloads  # noqa: F401
 from .fused_moe import (fused_experts, fused_experts_impl, fused_gate_topk, fused_topk,  # noqa: F401
-                        moe_align_block_size, quantize_expert_weights,
+                        fused_topk_experts, moe_align_block_size, quantize_expert_weights,
                         try_get_optimal_moe_config)
 from .layer import (FusedMoE, FusedMoEParallelConfig, MoEConfig, UnquantizedFusedMoEMethod,  # noqa: F401
                     Fp8E4M3FusedMoEMethod, GptOssMLP, RMSNorm, SparseMoeBlock)

@@ -31,6 +31,7 @@ EXPORTS = (
     "moe_align_can_plan", "moe_align_block_size_planned", "moe_fused_experts_plan_layout",
     "moe_fused_experts_status", "moe_fused_experts_set_wait_limit", "moe_align_block_size_static",
     "moe_tile_expert_weights", "moe_tile_expert_weights_supported",
+    "moe_route_align_supported", "moe_route_align_block_size",
 )
 
 
@@ -105,6 +106,10 @@ def _declare(L: ctypes.CDLL) -> None:
     L.moe_preferred_block_size.argtypes = [i32] * 5
     L.moe_quant_rows_e4m3.restype = i32
     L.moe_quant_rows_e4m3.argtypes = [p, i32, i64, i32, p, p, p]
+    L.moe_route_align_supported.restype = i32
+    L.moe_route_align_supported.argtypes = [i32, i32, i32]
+    L.moe_route_align_block_size.restype = i32
+    L.moe_route_align_block_size.argtypes = [p, p, p, p, i32, i32, i32, i32, i32, p, i64, p, i64, p, p, p, p, i32, i32]
     L.moe_tile_expert_weights_supported.restype = i32
     L.moe_tile_expert_weights_supported.argtypes = [i32] * 4
     L.moe_tile_expert_weights.restype = i32

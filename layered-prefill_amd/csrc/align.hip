@@ -16,10 +16,12 @@
 // the caller's workspace; three launches (count / scan / scatter) when the
 // tables of the second launch would not fit in LDS.
 #include "common.h"
+#include "routing_device.h"
 
 namespace {
 
 constexpr int kMaxExperts = 1024;
+constexpr int kRouteAlignMaxTokens = 512;       // rows the routing + alignment workgroup takes
 constexpr int kScanThreads = 1024;              // one thread per expert in the scans
 constexpr int kScanWaves = kScanThreads / kWave;
 constexpr int kSegLen = 512;                    // ids per wavefront segment, large path
@@ -191,12 +193,13 @@ __device__ void plan_from_counts(const volatile int* cum, const volatile int* to
   }
 }
 
-__global__ __launch_bounds__(kScanThreads) void align_small_kernel(
-    const void* __restrict__ ids, int dtype, int numel, int E, int BM, int id_bits,
-    int32_t* __restrict__ sorted_ids, int64_t sorted_cap, int32_t* __restrict__ expert_ids,
-    int64_t expert_cap, int32_t* __restrict__ num_post_pad, int32_t* plan_bounds, int32_t* plan_done,
-    int plan_num_done, int plan_cap_mb) {
-  extern __shared__ int lds[];
+// The single-workgroup alignment: histogram, scans and scatter in LDS (`lds`: kScanWaves * E +
+// 2 E + kScanWaves + 2 ints).  Called by all kScanThreads threads; contains barriers.
+__device__ void align_small_body(const void* __restrict__ ids, int dtype, int numel, int E, int BM, int id_bits,
+                                 int32_t* __restrict__ sorted_ids, int64_t sorted_cap,
+                                 int32_t* __restrict__ expert_ids, int64_t expert_cap,
+                                 int32_t* __restrict__ num_post_pad, int32_t* plan_bounds, int32_t* plan_done,
+                                 int plan_num_done, int plan_cap_mb, int* lds) {
   // layout: seg_cnt[kScanWaves][E] | cum[E+1] | tot[E] | wave_tot[kScanWaves+1]
   volatile int* seg_cnt = lds;
   volatile int* cum = lds + kScanWaves * E;
@@ -236,6 +239,63 @@ __global__ __launch_bounds__(kScanThreads) void align_small_kernel(
   // per-wavefront running slots: segment prefix + expert base
   for (int e = lane; e < E; e += kWave) seg_cnt[wave * E + e] += cum[e];
   scatter_segment(ids, dtype, beg, end, E, id_bits, seg_cnt + wave * E, sorted_ids);
+}
+
+__global__ __launch_bounds__(kScanThreads) void align_small_kernel(
+    const void* __restrict__ ids, int dtype, int numel, int E, int BM, int id_bits,
+    int32_t* __restrict__ sorted_ids, int64_t sorted_cap, int32_t* __restrict__ expert_ids,
+    int64_t expert_cap, int32_t* __restrict__ num_post_pad, int32_t* plan_bounds, int32_t* plan_done,
+    int plan_num_done, int plan_cap_mb) {
+  extern __shared__ int lds[];
+  align_small_body(ids, dtype, numel, E, BM, id_bits, sorted_ids, sorted_cap, expert_ids, expert_cap, num_post_pad,
+                   plan_bounds, plan_done, plan_num_done, plan_cap_mb, lds);
+}
+
+// Routing and alignment of a small batch in one launch (the decode-sized calls of a serving loop
+// are a handful of short kernels: every launch saved is several per cent of such a call).  The one
+// workgroup first routes all T rows, 16 wavefronts side by side with the lane layout, reduction
+// order and results of topk_softmax_pow2_kernel (csrc/moe_topk_softmax_kernels.cu:182-380 of the
+// reference), every row's loads issued before the first row is worked on; the ids it has written
+// are then aligned by the same code as align_small_kernel (stores of a workgroup are visible to
+// its own later loads behind a workgroup barrier).
+template <int E>
+__global__ __launch_bounds__(kScanThreads) void route_align_small_kernel(
+    const float* __restrict__ gating, float* __restrict__ topk_w, int32_t* __restrict__ topk_ids,
+    int32_t* __restrict__ tok_exp_idx, int T, int K, int renormalize, int BM, int id_bits,
+    int32_t* __restrict__ sorted_ids, int64_t sorted_cap, int32_t* __restrict__ expert_ids,
+    int64_t expert_cap, int32_t* __restrict__ num_post_pad, int32_t* plan_bounds, int32_t* plan_done,
+    int plan_num_done, int plan_cap_mb) {
+  extern __shared__ int lds[];
+  using G = Pow2Geom<E>;
+  constexpr int VPT = G::kVpt, TPR = G::kTpr, RPW = G::kRowsPerWave;
+  constexpr int kRowsPerPass = kScanWaves * RPW;   // rows the workgroup routes side by side
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int t = lane % TPR;
+  const int passes = (T + kRowsPerPass - 1) / kRowsPerPass;
+  // two passes in flight: the loads of pass i + 1 are issued before pass i is routed
+  float v[2][VPT];
+  auto row_of = [&](int pass) { return (pass * kScanWaves + wave) * RPW + lane / TPR; };
+  {
+    const int r = row_of(0);
+    load_row<E>(gating, r < T ? r : T - 1, t, v[0]);
+  }
+  for (int pass = 0; pass < passes; pass += 2) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int cur = pass + h;
+      if (cur < passes) {  // the same for every thread: whole wavefronts take part in the row's exchanges
+        if (cur + 1 < passes) {
+          const int rn = row_of(cur + 1);
+          load_row<E>(gating, rn < T ? rn : T - 1, t, v[h ^ 1]);
+        }
+        const int r = row_of(cur);
+        route_row<E>(v[h], t, r, r < T, topk_w, topk_ids, tok_exp_idx, T, K, renormalize);
+      }
+    }
+  }
+  __syncthreads();
+  align_small_body(topk_ids, MOE_ID_I32, T * K, E, BM, id_bits, sorted_ids, sorted_cap, expert_ids, expert_cap,
+                   num_post_pad, plan_bounds, plan_done, plan_num_done, plan_cap_mb, lds);
 }
 
 // ---- large path -----------------------------------------------------------
@@ -552,6 +612,61 @@ MOE_EXPORT int moe_align_block_size_planned(const void* topk_ids, int ids_dtype,
   return align_impl(topk_ids, ids_dtype, numel, E, block_size, sorted_token_ids, sorted_cap, expert_ids,
                     expert_cap, num_tokens_post_pad, workspace, workspace_bytes, stream, plan_bounds,
                     plan_done, plan_num_done, plan_cap_mb);
+}
+
+// Routing (moe_topk_softmax) and alignment (moe_align_block_size, with the plan of
+// moe_align_block_size_planned when plan_bounds is given) of a small batch as one launch.
+MOE_EXPORT int moe_route_align_supported(int T, int E, int K) {
+  if (T < 1 || T > kRouteAlignMaxTokens || E < 1 || E > 256 || (E & (E - 1)) != 0 || K < 1 || K > E) return 0;
+  return static_cast<int64_t>(T) * K <= kSmallNumel ? 1 : 0;
+}
+
+template <int E>
+static void launch_route_align(const float* g, float* w, int32_t* ids, int32_t* tei, int T, int K, int renorm, int BM,
+                               int32_t* sorted, int64_t sorted_cap, int32_t* eids, int64_t expert_cap, int32_t* npp,
+                               int32_t* pb, int32_t* pd, int pnd, int pcap, hipStream_t s) {
+  const size_t lds = (static_cast<size_t>(kScanWaves) * E + (E + 1) + E + kScanWaves + 1) * sizeof(int);
+  hipLaunchKernelGGL(route_align_small_kernel<E>, dim3(1), dim3(kScanThreads), lds, s, g, w, ids, tei, T, K, renorm, BM,
+                     bits_for(E), sorted, sorted_cap, eids, expert_cap, npp, pb, pd, pnd, pcap);
+}
+
+MOE_EXPORT int moe_route_align_block_size(const float* gating_output, float* topk_weights, int32_t* topk_ids,
+                                          int32_t* token_expert_indices, int T, int E, int K, int renormalize,
+                                          int block_size, int32_t* sorted_token_ids, int64_t sorted_cap,
+                                          int32_t* expert_ids, int64_t expert_cap, int32_t* num_tokens_post_pad,
+                                          void* stream, int32_t* plan_bounds, int32_t* plan_done, int plan_num_done,
+                                          int plan_cap_mb) {
+  if (!moe_route_align_supported(T, E, K))
+    return moe_fail(MOE_ERR_UNSUPPORTED, "route_align_block_size: T=%d E=%d K=%d (at most %d tokens, a power-of-two "
+                    "number of experts up to 256, T*K <= %lld); route and align apart", T, E, K, kRouteAlignMaxTokens,
+                    static_cast<long long>(kSmallNumel));
+  if (block_size < 1) return moe_fail(MOE_ERR_ARG, "route_align_block_size: block_size %d", block_size);
+  if (!gating_output || !topk_weights || !topk_ids || !token_expert_indices || !sorted_token_ids || !expert_ids ||
+      !num_tokens_post_pad)
+    return moe_fail(MOE_ERR_ARG, "route_align_block_size: null pointer");
+  if (plan_bounds && (block_size != kPlanBlock || !plan_done || plan_num_done < 0 || plan_cap_mb < 1))
+    return moe_fail(MOE_ERR_ARG, "route_align_block_size: a plan needs block_size %d and the plan buffers", kPlanBlock);
+  const int64_t need_sorted = static_cast<int64_t>(T) * K + static_cast<int64_t>(E) * (block_size - 1);
+  if (need_sorted > INT32_MAX) return moe_fail(MOE_ERR_ARG, "route_align_block_size: padded length overflows int32");
+  if (sorted_cap < need_sorted || expert_cap < (need_sorted + block_size - 1) / block_size)
+    return moe_fail(MOE_ERR_ARG, "route_align_block_size: sorted_token_ids holds %lld (needs %lld), expert_ids %lld "
+                    "(needs %lld)", static_cast<long long>(sorted_cap), static_cast<long long>(need_sorted),
+                    static_cast<long long>(expert_cap), static_cast<long long>((need_sorted + block_size - 1) / block_size));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define MOE_ROUTE_ALIGN_CASE(N)                                                                                        \
+  case N:                                                                                                              \
+    launch_route_align<N>(gating_output, topk_weights, topk_ids, token_expert_indices, T, K, renormalize, block_size,  \
+                          sorted_token_ids, sorted_cap, expert_ids, expert_cap, num_tokens_post_pad, plan_bounds,      \
+                          plan_done, plan_num_done, plan_cap_mb, s);                                                   \
+    break;
+  switch (E) {
+    MOE_ROUTE_ALIGN_CASE(1) MOE_ROUTE_ALIGN_CASE(2) MOE_ROUTE_ALIGN_CASE(4) MOE_ROUTE_ALIGN_CASE(8)
+    MOE_ROUTE_ALIGN_CASE(16) MOE_ROUTE_ALIGN_CASE(32) MOE_ROUTE_ALIGN_CASE(64) MOE_ROUTE_ALIGN_CASE(128)
+    MOE_ROUTE_ALIGN_CASE(256)
+    default: return moe_fail(MOE_ERR_UNSUPPORTED, "route_align_block_size: E=%d", E);
+  }
+#undef MOE_ROUTE_ALIGN_CASE
+  return moe_check_launch("route_align_block_size");
 }
 
 // ---------------------------------------------------------------------------

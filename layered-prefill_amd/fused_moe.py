@@ -46,6 +46,22 @@ def _align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: int,
     return sorted_ids, expert_ids, num_tokens_post_pad
 
 
+def _route_align_block_size(gating_output: torch.Tensor, renormalize: bool, topk_weights: torch.Tensor,
+                            topk_ids: torch.Tensor, block_size: int, num_experts: int, plan
+                            ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``fused_topk`` into ``topk_weights`` / ``topk_ids`` and ``moe_align_block_size`` on the
+    ids as one launch (``ops.route_align_block_size``)."""
+    dev = topk_ids.device
+    max_num_tokens_padded = topk_ids.numel() + num_experts * (block_size - 1)
+    sorted_ids = torch.empty((max_num_tokens_padded,), dtype=torch.int32, device=dev)
+    expert_ids = torch.empty((cdiv(max_num_tokens_padded, block_size),), dtype=torch.int32, device=dev)
+    num_tokens_post_pad = torch.empty((1), dtype=torch.int32, device=dev)
+    token_expert_indicies = torch.empty_like(topk_ids)
+    ops.route_align_block_size(topk_weights, topk_ids, token_expert_indicies, gating_output, renormalize,
+                               num_experts, block_size, sorted_ids, expert_ids, num_tokens_post_pad, plan)
+    return sorted_ids, expert_ids, num_tokens_post_pad
+
+
 def _plan_in_workspace(workspace: torch.Tensor, T: int, H: int, I: int, E: int, K: int, block_size: int,
                        act_code: int, weight_code: int, numel: int):
     """Where the alignment may leave the large-tile kernel's per-XCD ranges and
@@ -154,6 +170,35 @@ def fused_experts(hidden_states: torch.Tensor,
                               apply_router_weight_on_input, per_channel_quant, global_num_experts,
                               expert_map, w1_scale, w2_scale, w1_zp, w2_zp, a1_scale, a2_scale,
                               block_shape, w1_bias, w2_bias, weight_layout)
+
+
+def fused_topk_experts(hidden_states: torch.Tensor, gating_output: torch.Tensor, w1: torch.Tensor,
+                       w2: torch.Tensor, topk: int, renormalize: bool,
+                       w1_bias: Optional[torch.Tensor] = None, w2_bias: Optional[torch.Tensor] = None,
+                       inplace: bool = False, activation: str = "silu",
+                       apply_router_weight_on_input: bool = False,
+                       w1_scale: Optional[torch.Tensor] = None, w2_scale: Optional[torch.Tensor] = None,
+                       weight_layout: str = "plain") -> torch.Tensor:
+    """``fused_topk`` followed by ``fused_experts``: the two calls of
+    ``UnquantizedFusedMoEMethod.apply`` (nanovllm/layers/fused_moe.py:163-216) as one function, so
+    that for decode-sized batches (``ops.route_align_supported``) routing and alignment go out as
+    one launch instead of two.  Same result as the two calls, bit for bit."""
+    assert hidden_states.shape[0] == gating_output.shape[0], "Number of tokens mismatch"
+    M, E = gating_output.shape
+    if hidden_states.is_cuda and M > 0 and w1.size(0) == E and ops.route_align_supported(M, E, topk):
+        gating = gating_output if gating_output.dtype == torch.float32 else gating_output.float()
+        topk_weights = torch.empty(M, topk, dtype=torch.float32, device=hidden_states.device)
+        topk_ids = torch.empty(M, topk, dtype=torch.int32, device=hidden_states.device)
+        out = fused_experts_impl(hidden_states, w1, w2, topk_weights, topk_ids, inplace, activation,
+                                 apply_router_weight_on_input, w1_scale is not None, -1, None, w1_scale, w2_scale,
+                                 None, None, None, None, None, w1_bias, w2_bias, weight_layout,
+                                 _route=(gating.contiguous(), renormalize))
+        return hidden_states if inplace else out
+    topk_weights, topk_ids, _ = fused_topk(hidden_states, gating_output, topk, renormalize)
+    return fused_experts(hidden_states, w1, w2, w1_bias, w2_bias, topk_weights, topk_ids, inplace=inplace,
+                         activation=activation, apply_router_weight_on_input=apply_router_weight_on_input,
+                         per_channel_quant=w1_scale is not None, w1_scale=w1_scale, w2_scale=w2_scale,
+                         weight_layout=weight_layout)
 
 
 def fused_experts_workspace_bytes(tokens: int, hidden: int, intermediate: int, experts: int,
@@ -267,7 +312,7 @@ def fused_experts_impl(hidden_states: torch.Tensor,
                        block_shape: Optional[list] = None,
                        w1_bias: Optional[torch.Tensor] = None,
                        w2_bias: Optional[torch.Tensor] = None,
-                       weight_layout: str = "plain") -> torch.Tensor:
+                       weight_layout: str = "plain", _route=None) -> torch.Tensor:
     """nanovllm/layers/for_moe/fused_moe.py:461-633: align -> gate-up GEMM with
     the gated activation -> down GEMM times the routed weight -> top-k sum, in
     chunks of 64K tokens."""
@@ -361,8 +406,14 @@ def fused_experts_impl(hidden_states: torch.Tensor,
         if global_num_experts == E:
             plan = _plan_in_workspace(workspace, tokens_in_chunk, w1.size(2), N // 2, E, top_k_num, bm,
                                       act_code, weight_code, curr_ids.numel())
-        sorted_token_ids, expert_ids, num_tokens_post_padded = _align_block_size(
-            curr_ids, bm, global_num_experts, plan)
+        if _route is not None:
+            # routing and alignment as one launch (fused_topk_experts): topk_weights / topk_ids
+            # are this call's own buffers and are filled here, in front of their first use
+            sorted_token_ids, expert_ids, num_tokens_post_padded = _route_align_block_size(
+                _route[0], _route[1], curr_w, curr_ids, bm, global_num_experts, plan)
+        else:
+            sorted_token_ids, expert_ids, num_tokens_post_padded = _align_block_size(
+                curr_ids, bm, global_num_experts, plan)
         args = launch_fused_experts(hidden_states[begin:end], out_hidden_states[begin:end], w1, w2,
                                     w1_bias, w2_bias, w1_scale, w2_scale, curr_w, sorted_token_ids,
                                     expert_ids, num_tokens_post_padded, bm, activation,

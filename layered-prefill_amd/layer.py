@@ -16,7 +16,7 @@ import torch
 import torch.distributed as dist
 
 from . import ops
-from .fused_moe import fused_experts, fused_gate_topk, fused_topk
+from .fused_moe import fused_experts, fused_gate_topk, fused_topk, fused_topk_experts
 
 
 @dataclass
@@ -92,6 +92,18 @@ class UnquantizedFusedMoEMethod:
               expert_load_view: Optional[torch.Tensor] = None,
               logical_to_physical_map: Optional[torch.Tensor] = None,
               logical_replica_count: Optional[torch.Tensor] = None) -> torch.Tensor:
+        layout = "tiled" if getattr(layer, "weights_tiled", False) else "plain"
+        if (custom_routing_function is None and not use_grouped_topk and scoring_func == "softmax"
+                and e_score_correction_bias is None and expert_map is None
+                and self.topk_indices_dtype is None and self.fused_experts is fused_experts):
+            # plain softmax routing: select_experts + fused_experts as one function, which
+            # enqueues routing and alignment of a decode-sized batch as one launch
+            return fused_topk_experts(
+                x, router_logits, layer.w13_weight, layer.w2_weight, top_k, renormalize,
+                w1_bias=layer.w13_bias if hasattr(layer, "w13_bias") else None,
+                w2_bias=layer.w2_bias if hasattr(layer, "w2_bias") else None,
+                inplace=True, activation=activation,
+                apply_router_weight_on_input=apply_router_weight_on_input, weight_layout=layout)
         topk_weights, topk_ids = FusedMoE.select_experts(
             hidden_states=x, router_logits=router_logits, use_grouped_topk=use_grouped_topk,
             top_k=top_k, renormalize=renormalize, topk_group=topk_group,
@@ -104,8 +116,7 @@ class UnquantizedFusedMoEMethod:
             w2_bias=layer.w2_bias if hasattr(layer, "w2_bias") else None,
             topk_weights=topk_weights, topk_ids=topk_ids, inplace=True, activation=activation,
             apply_router_weight_on_input=apply_router_weight_on_input,
-            global_num_experts=global_num_experts, expert_map=expert_map,
-            weight_layout="tiled" if getattr(layer, "weights_tiled", False) else "plain")
+            global_num_experts=global_num_experts, expert_map=expert_map, weight_layout=layout)
 
     def process_weights_after_loading(self, layer: torch.nn.Module) -> None:
         """With ``FusedMoE(weight_layout="tiled")``: re-orders ``w13_weight`` and ``w2_weight`` once,

@@ -161,6 +161,49 @@ def align_block_size_planned(topk_ids: torch.Tensor, num_experts: int, block_siz
             check(L.moe_align_block_size_planned(*common, *plan))
 
 
+def route_align_supported(num_tokens: int, num_experts: int, topk: int) -> bool:
+    """Sizes ``route_align_block_size`` takes (a decode-sized batch, a power-of-two number of
+    experts up to 256)."""
+    return bool(lib().moe_route_align_supported(num_tokens, num_experts, topk))
+
+
+def route_align_block_size(topk_weights: torch.Tensor, topk_indices: torch.Tensor,
+                           token_expert_indices: torch.Tensor, gating_output: torch.Tensor,
+                           renormalize: bool, num_experts: int, block_size: int,
+                           sorted_token_ids: torch.Tensor, experts_ids: torch.Tensor,
+                           num_tokens_post_pad: torch.Tensor, plan=None) -> None:
+    """``topk_softmax`` (with the renormalisation of nanovllm/layers/for_moe/fused_moe.py:417-418)
+    and ``moe_align_block_size`` on its ids as one launch; ``plan`` as in
+    ``align_block_size_planned``.  Same results as the two ops, bit for bit.  No counterpart in the
+    reference, which enqueues them one after the other."""
+    require_gpu_tensor(gating_output, "gating_output")
+    if gating_output.dtype != torch.float32 or topk_weights.dtype != torch.float32:
+        raise RuntimeError("route_align_block_size: expected scalar type Float for gating_output / topk_weights")
+    for name, t in (("topk_indices", topk_indices), ("token_expert_indices", token_expert_indices),
+                    ("sorted_token_ids", sorted_token_ids), ("experts_ids", experts_ids),
+                    ("num_tokens_post_pad", num_tokens_post_pad)):
+        if t.dtype != torch.int32:
+            raise RuntimeError(f"route_align_block_size: {name} must be int32")
+    for name, t in (("topk_weights", topk_weights), ("topk_indices", topk_indices),
+                    ("token_expert_indices", token_expert_indices), ("gating_output", gating_output),
+                    ("sorted_token_ids", sorted_token_ids), ("experts_ids", experts_ids)):
+        if not t.is_contiguous():
+            raise RuntimeError(f"route_align_block_size: {name} must be contiguous")
+    T, E = gating_output.shape
+    K = topk_weights.size(-1)
+    if E != num_experts or topk_weights.numel() != T * K or topk_indices.numel() != T * K \
+            or token_expert_indices.numel() != T * K:
+        raise RuntimeError("route_align_block_size: output tensors must hold num_tokens * topk elements "
+                           "and gating_output num_experts columns")
+    pb, pd, pn, pc = plan if plan is not None else (None, None, 0, 0)
+    with torch.cuda.device(gating_output.device):
+        check(lib().moe_route_align_block_size(
+            gating_output.data_ptr(), topk_weights.data_ptr(), topk_indices.data_ptr(),
+            token_expert_indices.data_ptr(), T, E, K, int(renormalize), block_size,
+            sorted_token_ids.data_ptr(), sorted_token_ids.numel(), experts_ids.data_ptr(), experts_ids.numel(),
+            num_tokens_post_pad.data_ptr(), stream_ptr(gating_output.device), pb, pd, pn, pc))
+
+
 def _act_args(out: torch.Tensor, input: torch.Tensor):
     require_gpu_tensor(input, "input")
     if input.dtype not in _lib.DTYPE_CODE:

@@ -364,3 +364,64 @@ def test_planned_alignment_leaves_the_plan_of_the_plan_kernel(moe, oracle, dev, 
     live = int(got[2].item()) // 256
     assert bounds[0] == 0 and bounds[8] == live and bool((bounds[1:] >= bounds[:-1]).all())
     assert int((bounds[1:] - bounds[:-1]).max()) <= cap_mb
+
+
+@pytest.mark.parametrize("E,K", [(128, 8), (8, 2), (256, 6), (64, 1), (16, 16)])
+@pytest.mark.parametrize("T", [1, 37, 256, 512])
+@pytest.mark.parametrize("bm,renorm", [(32, True), (256, True), (64, False)])
+def test_route_align_one_launch_equals_the_two_ops(moe, oracle, dev, E, K, T, bm, renorm):
+    """``ops.route_align_block_size`` against the oracle's routing and alignment, bit for bit,
+    and against the two separate ops."""
+    print(f"route_align E={E} K={K} T={T} bm={bm}", flush=True)
+    g = torch.Generator().manual_seed(1000 * E + T)
+    logits = torch.randn(T, E, generator=g)
+    if T > 4:
+        logits[3] = logits[2]                      # equal rows route alike
+        logits[1] = torch.round(logits[1] * 4) / 4  # ties inside a row: lowest index first
+    ow, oids, otei = oracle.topk_softmax(logits, K, renormalize=renorm)
+    want = oracle.moe_align_block_size(oids, bm, E)
+    ld = logits.to(dev)
+    tw = torch.empty(T, K, dtype=torch.float32, device=dev)
+    ids = torch.empty(T, K, dtype=torch.int32, device=dev)
+    tei = torch.empty(T, K, dtype=torch.int32, device=dev)
+    cap = T * K + E * (bm - 1)
+    sorted_ids = torch.full((cap,), -7, dtype=torch.int32, device=dev)
+    expert_ids = torch.full((-(-cap // bm),), -7, dtype=torch.int32, device=dev)
+    npp = torch.full((1,), -7, dtype=torch.int32, device=dev)
+    assert moe.ops.route_align_supported(T, E, K)
+    moe.ops.route_align_block_size(tw, ids, tei, ld, renorm, E, bm, sorted_ids, expert_ids, npp)
+    torch.cuda.synchronize()
+    assert torch.equal(ids.cpu(), oids) and torch.equal(tei.cpu(), otei)
+    assert torch.equal(tw.cpu().view(torch.int32), ow.view(torch.int32))
+    for got, exp in zip((sorted_ids, expert_ids, npp), want):
+        assert torch.equal(got.cpu(), exp)
+
+
+def test_route_align_rejects_what_it_does_not_serve(moe, dev):
+    assert not moe.ops.route_align_supported(513, 128, 8)
+    assert not moe.ops.route_align_supported(64, 96, 8)      # not a power of two
+    assert not moe.ops.route_align_supported(512, 256, 64)   # T * K beyond the single-workgroup alignment
+    assert moe.ops.route_align_supported(512, 128, 8)
+
+
+@pytest.mark.parametrize("T", [64, 128, 256, 500])
+@pytest.mark.parametrize("layout", ["plain", "tiled"])
+def test_fused_topk_experts_equals_the_two_calls(moe, dev, T, layout):
+    """``fused_topk_experts`` (routing + alignment in one launch, with the large-tile plan at
+    256 tokens) gives the bits of ``fused_topk`` followed by ``fused_experts``."""
+    E, H, I, K = 128, 512, 256, 8
+    g = torch.Generator().manual_seed(T)
+    x = torch.randn(T, H, generator=g).bfloat16().to(dev)
+    logits = torch.randn(T, E, generator=g).to(dev)
+    w13 = (torch.randn(E, 2 * I, H, generator=g) * 0.02).bfloat16().to(dev)
+    w2 = (torch.randn(E, H, I, generator=g) * 0.02).bfloat16().to(dev)
+    if layout == "tiled":
+        w13, w2 = moe.ops.tile_expert_weights(w13, True), moe.ops.tile_expert_weights(w2, False)
+    tw, ids, _ = moe.fused_topk(x, logits, K, True)
+    two = moe.fused_experts(x, w13, w2, None, None, tw, ids, weight_layout=layout)
+    one = moe.fused_topk_experts(x, logits, w13, w2, K, True, weight_layout=layout)
+    torch.cuda.synchronize()
+    assert torch.equal(one.view(torch.int16), two.view(torch.int16))
+    xin = x.clone()
+    ret = moe.fused_topk_experts(xin, logits, w13, w2, K, True, inplace=True, weight_layout=layout)
+    assert ret is xin and torch.equal(xin.view(torch.int16), two.view(torch.int16))
