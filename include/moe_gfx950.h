@@ -131,13 +131,14 @@ int moe_align_block_size_planned(const void* topk_ids, int ids_dtype, int64_t nu
 
 
 /* moe_topk_softmax followed by moe_align_block_size (with the plan of
- * moe_align_block_size_planned when `plan_bounds` is not NULL) as ONE launch, for the small
+ * moe_align_block_size_planned when `plan_bounds` is not NULL) as ONE launch, for the smallest
  * batches of a decode loop: the reference enqueues these as two ops back to back
  * (nanovllm/layers/fused_moe.py:693-741 then nanovllm/layers/for_moe/fused_moe.py:575-577), each a
  * few microseconds, so every launch saved counts.  Results are those of the two calls, bit for bit:
  * `topk_ids` ([T, K] int32) is what gets aligned.  Served sizes (moe_route_align_supported returns
- * 1): T <= 512, E a power of two <= 256, K <= E, T * K <= 16384; otherwise MOE_ERR_UNSUPPORTED and
- * the caller routes and aligns apart.  No workspace. */
+ * 1): T <= 32 (one workgroup routes the rows: beyond 32 the two kernels, whose router spreads over
+ * the chip, are faster), E a power of two <= 256, K <= E; otherwise MOE_ERR_UNSUPPORTED and the
+ * caller routes and aligns apart.  No workspace. */
 int moe_route_align_supported(int T, int E, int K);
 int moe_route_align_block_size(const float* gating_output, float* topk_weights, int32_t* topk_ids,
                                int32_t* token_expert_indices, int T, int E, int K, int renormalize,

@@ -181,8 +181,8 @@ def fused_topk_experts(hidden_states: torch.Tensor, gating_output: torch.Tensor,
                        weight_layout: str = "plain") -> torch.Tensor:
     """``fused_topk`` followed by ``fused_experts``: the two calls of
     ``UnquantizedFusedMoEMethod.apply`` (nanovllm/layers/fused_moe.py:163-216) as one function, so
-    that for decode-sized batches (``ops.route_align_supported``) routing and alignment go out as
-    one launch instead of two.  Same result as the two calls, bit for bit."""
+    that for the smallest batches (``ops.route_align_supported``: up to 32 tokens) routing and
+    alignment go out as one launch instead of two.  Same result as the two calls, bit for bit."""
     assert hidden_states.shape[0] == gating_output.shape[0], "Number of tokens mismatch"
     M, E = gating_output.shape
     if hidden_states.is_cuda and M > 0 and w1.size(0) == E and ops.route_align_supported(M, E, topk):

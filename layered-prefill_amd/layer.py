@@ -97,7 +97,7 @@ class UnquantizedFusedMoEMethod:
                 and e_score_correction_bias is None and expert_map is None
                 and self.topk_indices_dtype is None and self.fused_experts is fused_experts):
             # plain softmax routing: select_experts + fused_experts as one function, which
-            # enqueues routing and alignment of a decode-sized batch as one launch
+            # enqueues routing and alignment of a batch of up to 32 tokens as one launch
             return fused_topk_experts(
                 x, router_logits, layer.w13_weight, layer.w2_weight, top_k, renormalize,
                 w1_bias=layer.w13_bias if hasattr(layer, "w13_bias") else None,

@@ -162,7 +162,7 @@ def align_block_size_planned(topk_ids: torch.Tensor, num_experts: int, block_siz
 
 
 def route_align_supported(num_tokens: int, num_experts: int, topk: int) -> bool:
-    """Sizes ``route_align_block_size`` takes (a decode-sized batch, a power-of-two number of
+    """Sizes ``route_align_block_size`` takes (at most 32 tokens, a power-of-two number of
     experts up to 256)."""
     return bool(lib().moe_route_align_supported(num_tokens, num_experts, topk))
 

@@ -367,7 +367,7 @@ def test_planned_alignment_leaves_the_plan_of_the_plan_kernel(moe, oracle, dev, 
 
 
 @pytest.mark.parametrize("E,K", [(128, 8), (8, 2), (256, 6), (64, 1), (16, 16)])
-@pytest.mark.parametrize("T", [1, 37, 256, 512])
+@pytest.mark.parametrize("T", [1, 7, 20, 32])
 @pytest.mark.parametrize("bm,renorm", [(32, True), (256, True), (64, False)])
 def test_route_align_one_launch_equals_the_two_ops(moe, oracle, dev, E, K, T, bm, renorm):
     """``ops.route_align_block_size`` against the oracle's routing and alignment, bit for bit,
@@ -398,18 +398,19 @@ def test_route_align_one_launch_equals_the_two_ops(moe, oracle, dev, E, K, T, bm
 
 
 def test_route_align_rejects_what_it_does_not_serve(moe, dev):
-    assert not moe.ops.route_align_supported(513, 128, 8)
-    assert not moe.ops.route_align_supported(64, 96, 8)      # not a power of two
-    assert not moe.ops.route_align_supported(512, 256, 64)   # T * K beyond the single-workgroup alignment
-    assert moe.ops.route_align_supported(512, 128, 8)
+    assert not moe.ops.route_align_supported(33, 128, 8)     # one workgroup routes 32 rows at most
+    assert not moe.ops.route_align_supported(16, 96, 8)      # not a power of two
+    assert not moe.ops.route_align_supported(16, 8, 9)       # top-k beyond the experts
+    assert moe.ops.route_align_supported(32, 128, 8)
 
 
-@pytest.mark.parametrize("T", [64, 128, 256, 500])
+@pytest.mark.parametrize("T", [5, 32, 64, 500])
 @pytest.mark.parametrize("layout", ["plain", "tiled"])
-def test_fused_topk_experts_equals_the_two_calls(moe, dev, T, layout):
-    """``fused_topk_experts`` (routing + alignment in one launch, with the large-tile plan at
-    256 tokens) gives the bits of ``fused_topk`` followed by ``fused_experts``."""
-    E, H, I, K = 128, 512, 256, 8
+@pytest.mark.parametrize("E,K", [(128, 8), (4, 4)])   # (4, 4) at 32 tokens: blocks of 256, the alignment also plans
+def test_fused_topk_experts_equals_the_two_calls(moe, dev, T, layout, E, K):
+    """``fused_topk_experts`` (routing + alignment in one launch up to 32 tokens, the two
+    calls beyond) gives the bits of ``fused_topk`` followed by ``fused_experts``."""
+    H, I = 512, 256
     g = torch.Generator().manual_seed(T)
     x = torch.randn(T, H, generator=g).bfloat16().to(dev)
     logits = torch.randn(T, E, generator=g).to(dev)
