@@ -213,7 +213,10 @@ typedef struct MoeFusedExpertsArgs {
      or benchmark time one pass alone (the later passes then read whatever the
      workspace holds).  Bit 8 keeps the two GEMM passes in separate launches
      where the library would otherwise enqueue them as one.  Bit 16: the
-     workspace already holds the plan (moe_align_block_size_planned). */
+     workspace already holds the plan (moe_align_block_size_planned).  Bit 32 (for
+     tests of the one-launch form): its down tiles run on the XCD next to the one
+     that ran their block's gate-up tiles, so every hand-off crosses two L2s; the
+     result is the same, bit for bit. */
   int32_t passes;
   int32_t weight_layout;     /* MoeWeightLayout of w13 and w2 (both): 0 = plain                   */
   void* stream;

@@ -1197,11 +1197,16 @@ __device__ __forceinline__ void big_poison_tile(const GemmParams& p, int mb, int
 template <typename Mma>
 __global__ __launch_bounds__(kThreads, 1) void big_fused_kernel(const GemmParams p1, const GemmParams p2,
                                                                 int32_t* __restrict__ done, int cap_mb,
-                                                                int spin_limit, int32_t* __restrict__ status) {
+                                                                int spin_limit, int32_t* __restrict__ status,
+                                                                int down_xcd_shift) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  const int x = blockIdx.x % kXcds, xslot = blockIdx.x / kXcds;
-  const int lo = p1.xcd_bounds[x], hi = p1.xcd_bounds[x + 1];
+  const int xslot = blockIdx.x / kXcds;
   const int n1 = cap_mb * p1.num_n_tiles;
+  // down_xcd_shift != 0 (a test setting): the down tiles of XCD x take the m-block range of XCD
+  // x + shift, so that every hand-off crosses from one XCD's L2 to another's.  Gate-up tiles never
+  // wait and precede the down tiles in every XCD's list, so the grid still drains.
+  const int x = (blockIdx.x % kXcds + (xslot < n1 ? 0 : down_xcd_shift)) % kXcds;
+  const int lo = p1.xcd_bounds[x], hi = p1.xcd_bounds[x + 1];
   if (xslot < n1) {
     const int mb = lo + xslot / p1.num_n_tiles, nt = xslot % p1.num_n_tiles;
     if (mb >= hi || lo < 0 || mb >= p1.num_m_blocks) return;  // (an unwritten plan must not send a tile out of range)
@@ -1227,17 +1232,20 @@ __global__ __launch_bounds__(kThreads, 1) void big_fused_kernel(const GemmParams
       while (!(ready = __hip_atomic_load(done + mb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= p1.num_n_tiles) &&
              spins++ < spin_limit)
         __builtin_amdgcn_s_sleep(32);
-      // loads of the block's rows come after the full count was seen (drops this CU's cached lines)
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
       *s_flag = ready ? 1 : 0;
     }
     __syncthreads();
+    // Every wavefront orders its own loads of the block's rows behind the count it has just been told
+    // of: the acquire fence drops the cached lines (and completes, vmcnt(0)) in the wavefront that
+    // issues it, and a workgroup barrier alone does not extend that to the other three.
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     if (*s_flag == 0) {  // workgroup-uniform
       big_poison_tile<typename Mma::El>(p2, mb, nt);
       if (threadIdx.x == 0) __hip_atomic_fetch_add(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       return;
     }
-    // (the flag word lies in ring slot 4, which big_tile writes only behind its own barriers)
+    // (the flag word lies behind the epilogue's staging area and side arrays, in the ring's last unit,
+    // which big_tile writes only behind its own barriers)
     big_tile<Mma, false>(p2, mb, nt, smem);
   }
 }
@@ -1632,7 +1640,7 @@ static bool big_16bit_ok(const GemmParams& p, bool gated, int block_size, int64_
 // p1.xcd_bounds must be set; `done` holds one zeroed counter per m-block.
 template <typename Mma>
 int launch_big_fused(GemmParams& p1, GemmParams& p2, int block_size, int64_t sorted_cap, int32_t* done,
-                     int32_t* status, hipStream_t s) {
+                     int32_t* status, int down_xcd_shift, hipStream_t s) {
   constexpr int lds = kBigLdsTotal;
   auto kern = big_fused_kernel<Mma>;
   static MoeLdsOptIn opted;
@@ -1650,7 +1658,7 @@ int launch_big_fused(GemmParams& p1, GemmParams& p2, int block_size, int64_t sor
   const int64_t grid = static_cast<int64_t>(cap_mb) * (p1.num_n_tiles + p2.num_n_tiles) * kXcds;
   if (grid > INT32_MAX) return moe_fail(MOE_ERR_ARG, "fused_experts: grid of %lld workgroups", static_cast<long long>(grid));
   hipLaunchKernelGGL(kern, dim3(static_cast<unsigned>(grid)), dim3(kThreads), lds, s, p1, p2, done, cap_mb,
-                     g_wait_limit.load(std::memory_order_relaxed), status);
+                     g_wait_limit.load(std::memory_order_relaxed), status, down_xcd_shift);
   return moe_check_launch("fused_experts (gate-up and down pass, one launch)");
 }
 
@@ -1839,10 +1847,14 @@ static int check_fused_args(const MoeFusedExpertsArgs* a, int64_t* cap, int64_t*
     return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: e4m3 path needs H, I and weight strides in multiples of 16");
   if (a->activation < MOE_ACT_SILU || a->activation > MOE_ACT_GELU)
     return moe_fail(MOE_ERR_ARG, "fused_experts: unknown activation code %d", a->activation);
-  if (a->H % 8 || a->I % 8)
-    return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: H=%d and I=%d must be multiples of 8", a->H, a->I);
-  if (a->w13_stride_n % 8 || a->w13_stride_e % 8 || a->w2_stride_n % 8 || a->w2_stride_e % 8)
-    return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: weight strides must be multiples of 8 elements");
+  // rows move in 16-byte chunks: 8 elements of 16 bits, 4 of fp32 (16 of e4m3: checked above)
+  const int chunk = a->act_dtype == MOE_F32 ? 4 : 8;
+  if (a->H % chunk || a->I % chunk)
+    return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: H=%d and I=%d must be multiples of %d", a->H, a->I, chunk);
+  // (the expert stride of a single expert carries no meaning)
+  if (a->w13_stride_n % chunk || a->w2_stride_n % chunk ||
+      (a->E > 1 && (a->w13_stride_e % chunk || a->w2_stride_e % chunk)))
+    return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: weight strides must be multiples of %d elements", chunk);
   if ((reinterpret_cast<uintptr_t>(a->x) | reinterpret_cast<uintptr_t>(a->w13) |
        reinterpret_cast<uintptr_t>(a->w2) | reinterpret_cast<uintptr_t>(a->out)) & 15u)
     return moe_fail(MOE_ERR_ARG, "fused_experts: tensors must be 16-byte aligned");
@@ -1988,8 +2000,9 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
     p2.c_tiled = 0; p2.a_tiled = inter_tiled ? 1 : 0;
     if (big_16bit_ok(p, true, a->block_size, cap) && big_16bit_ok(p2, false, a->block_size, cap)) {
       int32_t* status = const_cast<int32_t*>(plan_bounds) + kBigStatusWord;
-      rc = a->act_dtype == MOE_BF16 ? launch_big_fused<MmaBF16>(p, p2, a->block_size, cap, plan_done, status, s)
-                                    : launch_big_fused<MmaF16>(p, p2, a->block_size, cap, plan_done, status, s);
+      const int shift = (a->passes & 32) ? 1 : 0;  // test setting: every hand-off crosses XCDs
+      rc = a->act_dtype == MOE_BF16 ? launch_big_fused<MmaBF16>(p, p2, a->block_size, cap, plan_done, status, shift, s)
+                                    : launch_big_fused<MmaF16>(p, p2, a->block_size, cap, plan_done, status, shift, s);
       if (rc) return rc;
       if (!(passes & 4)) return MOE_OK;
       return moe_sum(a->out, c3, a->T, a->K, a->H, a->act_dtype, a->stream);

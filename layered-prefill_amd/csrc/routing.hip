@@ -326,7 +326,10 @@ __global__ __launch_bounds__(kWave) void topk_softmax_wide_kernel(
 
   float wsum = 0.f;
   for (int k = 0; k < K; ++k) {
-    float best = -20000.f;  // below the marker of a taken column
+    // below the marker of a taken column.  (A row with fewer than K comparable probabilities, i.e.
+    // NaN logits, lets a taken column win again: the reference's fallback kernel behaves the same,
+    // csrc/moe_topk_softmax_kernels.cu:117-150, and such rows carry no meaning.)
+    float best = -20000.f;
     int bidx = lane;
     for (int c = lane; c < E; c += kWave) {
       const float v = prob[c];
@@ -375,6 +378,10 @@ MOE_EXPORT int moe_topk_softmax(const float* gating_output, float* topk_weights,
     return moe_fail(MOE_ERR_UNSUPPORTED, "topk_softmax: num_experts %d > %d", E, kWideMaxExperts);
   if (static_cast<int64_t>(T) * K > INT32_MAX)
     return moe_fail(MOE_ERR_ARG, "topk_softmax: T*K overflows int32 token_expert_indices");
+  // one 64-lane workgroup per row beyond 1024 experts: the grid's thread count has to fit 32 bits
+  if (E > kWave * kGenericMaxPerLane && static_cast<int64_t>(T) > (static_cast<int64_t>(UINT32_MAX) / kWave))
+    return moe_fail(MOE_ERR_UNSUPPORTED, "topk_softmax: %d rows of %d experts exceed the launch limit of %lld rows", T, E,
+                    static_cast<long long>(UINT32_MAX / kWave));
   if (T == 0) return MOE_OK;
   if (!gating_output || !topk_weights || !topk_ids || !token_expert_indices)
     return moe_fail(MOE_ERR_ARG, "topk_softmax: null pointer");

@@ -154,6 +154,16 @@ def test_fused_experts_states_its_narrower_contract(moe):
     w1 = torch.zeros(2, 32, 68, dtype=torch.bfloat16)[:, :, :64]      # row stride 68
     with pytest.raises(AssertionError, match="weight strides"):
         moe.fused_experts(x, w1, torch.zeros(2, 64, 16, dtype=torch.bfloat16), None, None, tw, ids)
+    # 16 bytes are four fp32 elements: H = 60 passes the size rule in fp32 (and stops at the device check)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        moe.fused_experts(torch.zeros(4, 60), torch.zeros(2, 24, 60), torch.zeros(2, 60, 12), None, None, tw, ids)
+    with pytest.raises(AssertionError, match="multiples of 4"):
+        moe.fused_experts(torch.zeros(4, 62), torch.zeros(2, 24, 62), torch.zeros(2, 62, 12), None, None, tw, ids)
+    # the stride of a dimension of size 1 says nothing: one expert cut out of a larger tensor
+    one13 = torch.zeros(3, 32, 64, dtype=torch.bfloat16).as_strided((1, 32, 64), (2051, 64, 1))
+    one2 = torch.zeros(3, 64, 16, dtype=torch.bfloat16)[:1]
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        moe.fused_experts(x, one13, one2, None, None, tw, torch.zeros(4, 2, dtype=torch.int32))
     with pytest.raises(AssertionError, match="global_num_experts"):
         moe.fused_experts(x, torch.zeros(2, 32, 64, dtype=torch.bfloat16), torch.zeros(2, 64, 16, dtype=torch.bfloat16),
                           None, None, tw, ids, global_num_experts=4)

@@ -283,6 +283,52 @@ def test_swigluoai_matches_formula(oracle):
     assert torch.allclose(out.double(), ref, rtol=3e-6, atol=1e-6)
 
 
+def _ulp_steps(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """Distance of two 16-bit tensors in representable values (same sign assumed where they differ)."""
+    ia, ib = a.view(torch.int16).int(), b.view(torch.int16).int()
+    return (ia - ib).abs()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_swigluoai_16bit_is_the_float64_formula_rounded_once(oracle, dtype):
+    """The bf16 branch (C) and the fp16 branch (Python) of ``swigluoai_and_mul`` have their own
+    interleave indexing: gate = even column, up = odd column, both clamps, one rounding at the
+    end.  Against the closed form in float64 rounded once; swapping even and odd, dropping a
+    clamp or rounding an intermediate fails it."""
+    x = (torch.randn(29, 2 * 48, generator=torch.Generator().manual_seed(8)) * 5).to(dtype)
+    out = oracle.swigluoai_and_mul(x, 1.702, 7.0)
+    assert out.dtype == dtype and tuple(out.shape) == (29, 48)
+    g = x[:, 0::2].double().clamp(max=7.0)
+    u = x[:, 1::2].double().clamp(-7.0, 7.0)
+    ref = ((u + 1) * g * torch.sigmoid(1.702 * g)).to(dtype)
+    steps = _ulp_steps(out, ref)
+    assert int(steps.max()) <= 1                    # fp32 evaluation against float64: a rounding tie at most
+    assert (steps > 0).float().mean() < 0.01
+    assert (x[:, 0::2].float() > 7).any() and (x[:, 1::2].float().abs() > 7).any()   # the clamps were exercised
+    swapped = ((g + 1) * u.clamp(max=7.0) * torch.sigmoid(1.702 * u)).to(dtype)       # even/odd exchanged
+    assert int(_ulp_steps(out, swapped).max()) > 1
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_gelu_and_mul_16bit_rounds_the_activation_then_the_product(oracle, dtype):
+    """nanovllm/layers/for_moe/moe_easy_kernel.py:89-98 in a 16-bit dtype: erf GELU of the first
+    half rounded to the dtype, times the second half, rounded again."""
+    x = (torch.randn(31, 2 * 40, generator=torch.Generator().manual_seed(9)) * 3).to(dtype)
+    out = oracle.gelu_and_mul(x)
+    g, u = x[:, :40].double(), x[:, 40:].double()
+    act = (0.5 * g * (1 + torch.erf(g / 2 ** 0.5))).to(dtype)
+    ref = (act.double() * u).to(dtype)
+    # (far in the negative tail 1 + erf cancels in fp32: there the values are below 1e-5 and only
+    # their absolute distance says anything)
+    steps = _ulp_steps(out, ref)
+    tail = (out.double() - ref.double()).abs() < 1e-5
+    assert bool(((steps <= 1) | tail).all()) and ((steps > 0) & ~tail).float().mean() < 0.01
+    halves_swapped = ((0.5 * u * (1 + torch.erf(u / 2 ** 0.5))).to(dtype).double() * g).to(dtype)
+    assert int(_ulp_steps(out, halves_swapped).max()) > 1
+    once = (0.5 * g * (1 + torch.erf(g / 2 ** 0.5)) * u).to(dtype)                    # a single rounding differs somewhere
+    assert not torch.equal(out, once)
+
+
 # ----------------------------------------------------------------- fp8 helpers
 def test_e4m3_quantiser_matches_torch_cast_and_saturates(oracle):
     x = torch.cat([torch.linspace(-448, 448, 100001), torch.tensor([0.0, 1e-4, 2 ** -9, 2 ** -10,
@@ -560,6 +606,37 @@ def test_mirror_rounding_step_by_step_on_a_2x2_case(oracle):
     want32 = torch.stack([(silu(gate32) * up32 * w2f[0, r, 0]) * tw[0, 0] for r in range(2)])
     got32 = oracle.fused_experts_ref(x, w13, w2, tw, ids)
     assert torch.allclose(got32[0], want32, rtol=1e-6, atol=0) and not torch.equal(got32, got_fused)
+
+
+def test_mirror_rounding_step_by_step_gelu_and_swigluoai(oracle):
+    """The mirrored mode with the other two activations on the same hand-sized case: GEMM1
+    rounded, the activation rounded where the reference's kernels round it (gelu: activation,
+    then product; swigluoai: once, gate = row 0 and up = row 1 of the interleaved pair), weighted
+    GEMM2 rounded, sum rounded."""
+    x = torch.tensor([[1.5390625, -0.29296875]]).bfloat16()
+    w13 = torch.tensor([[[-2.171875, 0.5703125], [-1.0859375, -1.3984375]]]).bfloat16()
+    w2 = torch.tensor([[[0.404296875], [0.83984375]]]).bfloat16()
+    tw = torch.tensor([[0.7]])
+    ids = torch.zeros(1, 1, dtype=torch.int32)
+    xf, w13f, w2f = x.float(), w13.float(), w2.float()
+    r0 = _bf(xf[0, 0] * w13f[0, 0, 0] + xf[0, 1] * w13f[0, 0, 1])    # row 0 of w13 after GEMM1, rounded
+    r1 = _bf(xf[0, 0] * w13f[0, 1, 0] + xf[0, 1] * w13f[0, 1, 1])    # row 1
+    finish = lambda c2: torch.stack([_bf(_bf((c2 * w2f[0, r, 0]) * tw[0, 0])) for r in range(2)])
+    # gelu: halves layout (I = 1: row 0 gate, row 1 up); erf form in float64, rounded, product rounded
+    act = _bf(0.5 * r0.double() * (1 + torch.erf(r0.double() / 2 ** 0.5)))
+    c2 = _bf(act * r1)
+    assert c2 != act * r1 or act != 0.5 * r0 * (1 + torch.erf(r0 / 2 ** 0.5))   # a rounding bites
+    got = oracle.fused_experts_ref(x, w13, w2, tw, ids, activation="gelu", mirror_rounding=True)
+    assert torch.equal(got[0], finish(c2))
+    # swigluoai: interleaved pair (row 0 gate, row 1 up), clamps inactive here, one rounding
+    a, lim = 1.702, 7.0
+    g64, u64 = r0.double().clamp(max=lim), r1.double().clamp(-lim, lim)
+    c2s = _bf((u64 + 1) * g64 * torch.sigmoid(a * g64))
+    got = oracle.fused_experts_ref(x, w13, w2, tw, ids, activation="swigluoai", mirror_rounding=True)
+    assert torch.equal(got[0], finish(c2s))
+    # gate and up exchanged would be another number
+    c2x = _bf((g64 + 1) * u64.clamp(max=lim) * torch.sigmoid(a * u64))
+    assert not torch.equal(finish(c2x), finish(c2s))
 
 
 # ----------------------------------------------------------------- fp8 expert MLP
