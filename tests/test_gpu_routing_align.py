@@ -426,3 +426,35 @@ def test_fused_topk_experts_equals_the_two_calls(moe, dev, T, layout, E, K):
     xin = x.clone()
     ret = moe.fused_topk_experts(xin, logits, w13, w2, K, True, inplace=True, weight_layout=layout)
     assert ret is xin and torch.equal(xin.view(torch.int16), two.view(torch.int16))
+
+
+def test_fused_topk_experts_inside_a_hip_graph(moe, dev):
+    """A call made while the stream is captured enqueues the two kernels (routing, alignment)
+    instead of the one launch; every replay gives the bits of the eager call, with eager
+    work and synchronisations of the program's own between the replays."""
+    T, H, I, E, K = 16, 512, 256, 128, 8
+    g = torch.Generator().manual_seed(16)
+    x = torch.randn(T, H, generator=g).bfloat16().to(dev)
+    logits = torch.randn(T, E, generator=g).to(dev)
+    w13 = (torch.randn(E, 2 * I, H, generator=g) * 0.02).bfloat16().to(dev)
+    w2 = (torch.randn(E, H, I, generator=g) * 0.02).bfloat16().to(dev)
+    assert moe.ops.route_align_supported(T, E, K)
+    eager = moe.fused_topk_experts(x, logits, w13, w2, K, True)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        moe.fused_topk_experts(x, logits, w13, w2, K, True)   # warm-up on the capture stream
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            captured = moe.fused_topk_experts(x, logits, w13, w2, K, True)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        captured.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(captured.view(torch.int16), eager.view(torch.int16)), rep
+        again = moe.fused_topk_experts(x, logits, w13, w2, K, True)   # eager work between replays
+        torch.cuda.synchronize()
+        assert torch.equal(again.view(torch.int16), eager.view(torch.int16))
