@@ -174,7 +174,12 @@ int moe_sum(void* out, const void* in, int64_t T, int K, int H, int dtype, void*
  * (nanovllm/layers/for_moe/fused_moe.py:579-631): grouped GEMM x*W13^T with the
  * gated activation fused into its epilogue, grouped GEMM with W2^T times the
  * routed weight, and the top-k combine.  `out` may alias `x` (inplace=True at
- * nanovllm/layers/fused_moe.py:203-216). */
+ * nanovllm/layers/fused_moe.py:203-216).  Any H and I with bf16, fp16 and fp32 weights, as the
+ * Triton kernel's K and N masks allow (for_moe/fused_moe.py:191-205,218-223): the tuned kernels
+ * move rows in 16-byte chunks, and a call whose H, I or weight strides are not multiples of 16
+ * bytes, or whose tensors are only element-aligned, runs both GEMM passes on an
+ * element-by-element variant of the register-staged kernel (correct, untuned; plain weight
+ * layout only).  e4m3 weights: H, I and strides multiples of 16, tensors 16-byte aligned. */
 typedef struct MoeFusedExpertsArgs {
   /* tensors */
   const void* x;             /* [T, H] activations, row-major contiguous            */

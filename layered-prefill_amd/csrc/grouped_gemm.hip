@@ -135,6 +135,8 @@ struct GemmParams {
   int w_tiled;       // weights: units [expert][n-tile][K tile] (moe_tile_expert_weights)
   int a_tiled;       // A operand of the down pass: units [m-block][K tile]
   int c_tiled;       // result of the gate-up pass written as such units
+  int ragged;        // rows are not whole 16-byte chunks (K or a stride not a multiple of 16 bytes, or a
+                     // base that is not 16-byte aligned): the register-staged kernel loads element by element
 };
 
 constexpr int kThreads = 256;
@@ -217,7 +219,27 @@ __device__ __forceinline__ void store_fragment(const GemmParams& p, int e, const
   }
 }
 
-template <typename Mma, int BM, int BNW, int WAVES_M, bool GATED>
+// One 16-byte chunk of a row whose start is only element-aligned and of which only the first
+// `valid` elements exist (the rest reads as zero): what the Triton kernel of the reference does with
+// its K mask (nanovllm/layers/for_moe/fused_moe.py:191-205,218-223).
+template <int ES>
+__device__ __forceinline__ uint4 load_chunk_by_element(const char* ptr, int valid) {
+  uint32_t w[4] = {0, 0, 0, 0};
+  if constexpr (ES == 4) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < valid) w[i] = reinterpret_cast<const uint32_t*>(ptr)[i];
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (i < valid) w[i >> 1] |= static_cast<uint32_t>(reinterpret_cast<const uint16_t*>(ptr)[i]) << (16 * (i & 1));
+  }
+  return uint4{w[0], w[1], w[2], w[3]};
+}
+
+// RAGGED: operand rows are read element by element with a mask on K (any H, I, stride and
+// element-aligned base); the results are those of the 16-byte path wherever both apply.
+template <typename Mma, int BM, int BNW, int WAVES_M, bool GATED, bool RAGGED = false>
 __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams p) {
   using El = typename Mma::El;
   constexpr int ES = Mma::kEs;               // bytes per input element
@@ -321,6 +343,15 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
   const int nk = (p.Kd + BKE - 1) / BKE;
 
   auto gload = [&](int kt) {
+    if constexpr (RAGGED) {
+      static_assert(ES != 1, "e4m3 rows are whole 16-byte chunks");
+      const int valid = p.Kd - (kt * BKE + ld_c * CE);
+#pragma unroll
+      for (int j = 0; j < A_LD; ++j) a_reg[j] = load_chunk_by_element<ES>(a_src[j] + kt * kRowBytes, valid);
+#pragma unroll
+      for (int j = 0; j < B_LD; ++j) b_reg[j] = load_chunk_by_element<ES>(w_src[j] + kt * kRowBytes, valid);
+      return;
+    }
     const bool in_k = kt * BKE + ld_c * CE < p.Kd;
 #pragma unroll
     for (int j = 0; j < A_LD; ++j)
@@ -1604,10 +1635,10 @@ int launch_big(GemmParams& p, int64_t sorted_cap, hipStream_t s) {
   return moe_check_launch(GATED ? "fused_experts (gate-up pass)" : "fused_experts (down pass)");
 }
 
-template <typename Mma, int BM, int BNW, int WAVES_M, bool GATED>
+template <typename Mma, int BM, int BNW, int WAVES_M, bool GATED, bool RAGGED = false>
 int launch(const GemmParams& p, hipStream_t s) {
   constexpr int lds = 2 * (BM + BNW) * kRowBytes;
-  auto kern = grouped_gemm_kernel<Mma, BM, BNW, WAVES_M, GATED>;
+  auto kern = grouped_gemm_kernel<Mma, BM, BNW, WAVES_M, GATED, RAGGED>;
   static MoeLdsOptIn opted;  // per instantiation
   if (int rc = moe_opt_in_lds(opted, reinterpret_cast<const void*>(kern), lds, "fused_experts")) return rc;
   const int64_t tiles = static_cast<int64_t>(p.num_m_blocks) * p.num_n_tiles;
@@ -1668,6 +1699,16 @@ int launch_bm(GemmParams& p, int block_size, int64_t sorted_cap, hipStream_t s) 
   p.m_major = 0;
   const int32_t* bounds = p.xcd_bounds;  // meant for the large-tile kernel only
   p.xcd_bounds = nullptr;
+  if constexpr (Mma::kEs != 1) {
+    if (p.ragged) {
+      // any alignment block is a whole number of 32-slot tiles
+      if (block_size % 32 != 0)
+        return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: block_size %d is not a multiple of 32", block_size);
+      p.num_m_blocks = static_cast<int>((sorted_cap + 31) / 32);
+      p.num_n_tiles = (p.N + (GATED ? 128 : 256) - 1) / (GATED ? 128 : 256);
+      return launch<Mma, 32, 256, 1, GATED, true>(p, s);
+    }
+  }
   const bool offsets_fit = dma_offsets_fit(p, GATED, sorted_cap, Mma::kEs);
   if constexpr (Mma::kEs == 1) {
     // a large-tile K step is 128 bytes per row: 128 e4m3 elements
@@ -1825,6 +1866,17 @@ MOE_EXPORT int moe_fused_experts_plan_layout(int T, int H, int I, int E, int K, 
 // alignment of T * K ids over E experts can exceed.  A longer buffer is accepted and its
 // surplus ignored: every region of the workspace is laid out from `cap`, never from the
 // caller's figure.
+// Whether a 16-bit or fp32 call has rows that are not whole, aligned 16-byte chunks: H or I, a
+// weight stride (the expert stride of a single expert carries no meaning) or a base address.
+static bool fused_args_ragged(const MoeFusedExpertsArgs* a) {
+  if (a->weight_dtype == MOE_E4M3) return false;
+  const int chunk = a->act_dtype == MOE_F32 ? 4 : 8;
+  if (a->H % chunk || a->I % chunk || a->w13_stride_n % chunk || a->w2_stride_n % chunk) return true;
+  if (a->E > 1 && (a->w13_stride_e % chunk || a->w2_stride_e % chunk)) return true;
+  return ((reinterpret_cast<uintptr_t>(a->x) | reinterpret_cast<uintptr_t>(a->w13) |
+           reinterpret_cast<uintptr_t>(a->w2) | reinterpret_cast<uintptr_t>(a->out)) & 15u) != 0;
+}
+
 static int check_fused_args(const MoeFusedExpertsArgs* a, int64_t* cap, int64_t* need_ws) {
   if (!a) return moe_fail(MOE_ERR_ARG, "fused_experts: null argument block");
   if (a->T < 0 || a->H < 1 || a->I < 1 || a->E < 1 || a->K < 1 || a->block_size < 1)
@@ -1847,20 +1899,19 @@ static int check_fused_args(const MoeFusedExpertsArgs* a, int64_t* cap, int64_t*
     return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: e4m3 path needs H, I and weight strides in multiples of 16");
   if (a->activation < MOE_ACT_SILU || a->activation > MOE_ACT_GELU)
     return moe_fail(MOE_ERR_ARG, "fused_experts: unknown activation code %d", a->activation);
-  // rows move in 16-byte chunks: 8 elements of 16 bits, 4 of fp32 (16 of e4m3: checked above)
-  const int chunk = a->act_dtype == MOE_F32 ? 4 : 8;
-  if (a->H % chunk || a->I % chunk)
-    return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: H=%d and I=%d must be multiples of %d", a->H, a->I, chunk);
-  // (the expert stride of a single expert carries no meaning)
-  if (a->w13_stride_n % chunk || a->w2_stride_n % chunk ||
-      (a->E > 1 && (a->w13_stride_e % chunk || a->w2_stride_e % chunk)))
-    return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: weight strides must be multiples of %d elements", chunk);
-  if ((reinterpret_cast<uintptr_t>(a->x) | reinterpret_cast<uintptr_t>(a->w13) |
-       reinterpret_cast<uintptr_t>(a->w2) | reinterpret_cast<uintptr_t>(a->out)) & 15u)
-    return moe_fail(MOE_ERR_ARG, "fused_experts: tensors must be 16-byte aligned");
+  // Rows normally move in 16-byte chunks (8 elements of 16 bits, 4 of fp32).  Sizes, strides or
+  // bases that do not allow that take the element-by-element kernel (fused_args_ragged); e4m3 rows
+  // are always whole chunks (checked above), and so are their bases:
+  const uintptr_t bases = reinterpret_cast<uintptr_t>(a->x) | reinterpret_cast<uintptr_t>(a->w13) |
+                          reinterpret_cast<uintptr_t>(a->w2) | reinterpret_cast<uintptr_t>(a->out);
+  if (fp8 && (bases & 15u)) return moe_fail(MOE_ERR_ARG, "fused_experts: tensors must be 16-byte aligned");
+  if (bases & (a->act_dtype == MOE_F32 ? 3u : 1u))
+    return moe_fail(MOE_ERR_ARG, "fused_experts: tensors must be aligned to their element size");
   if (a->weight_layout != MOE_WEIGHTS_PLAIN && a->weight_layout != MOE_WEIGHTS_TILED)
     return moe_fail(MOE_ERR_ARG, "fused_experts: unknown weight_layout %d", a->weight_layout);
   if (a->weight_layout == MOE_WEIGHTS_TILED) {
+    if (fused_args_ragged(a))
+      return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: tiled weights need 16-byte aligned tensors");
     if (fp8 || a->act_dtype == MOE_F32)
       return moe_fail(MOE_ERR_UNSUPPORTED, "fused_experts: tiled weights are for bf16 and fp16 only");
     if (!moe_tile_expert_weights_supported(2 * a->I, a->H, 2, 1) || !moe_tile_expert_weights_supported(a->H, a->I, 2, 0))
@@ -1893,6 +1944,7 @@ static int check_fused_args(const MoeFusedExpertsArgs* a, int64_t* cap, int64_t*
 // intermediate as 32 KB units in the workspace (I a multiple of 64 is part of big_16bit_ok).
 static bool inter_units_ok(const MoeFusedExpertsArgs* a, int64_t cap) {
   if (a->block_size % kBigBM != 0 || a->act_dtype == MOE_F32 || a->weight_dtype == MOE_E4M3) return false;
+  if (fused_args_ragged(a)) return false;
   GemmParams p1{}, p2{};
   p1.numel = p2.numel = static_cast<int>(static_cast<int64_t>(a->T) * a->K);
   p1.top_k = p2.top_k = a->K;
@@ -1961,6 +2013,7 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   p.activation = a->activation;
   p.interleaved = a->activation == MOE_ACT_SWIGLUOAI;
   p.w_tiled = a->weight_layout == MOE_WEIGHTS_TILED ? 1 : 0;
+  p.ragged = fused_args_ragged(a) ? 1 : 0;
   const int32_t* plan_bounds = nullptr;
   int32_t* plan_done = nullptr;
   if (a->block_size % kBigBM == 0 && a->act_dtype != MOE_F32) {
@@ -1990,7 +2043,7 @@ MOE_EXPORT int moe_fused_experts(const MoeFusedExpertsArgs* a) {
   // sizes only, never on `passes`, so single passes enqueued apart agree on it.
   const bool inter_tiled = plan_bounds && !fp8 && inter_units_ok(a, cap);
   p.c_tiled = inter_tiled ? 1 : 0;
-  if (plan_bounds && !fp8 && (passes & 3) == 3 && !(passes & 8)) {
+  if (plan_bounds && !fp8 && !p.ragged && (passes & 3) == 3 && !(passes & 8)) {
     // 16-bit dtypes on the large-tile kernel: both passes in one launch
     GemmParams p2 = p;
     p2.a = inter; p2.lda = a->I; p2.w = a->w2; p2.w_stride_e = a->w2_stride_e; p2.w_stride_n = a->w2_stride_n;

@@ -363,16 +363,18 @@ def fused_experts_impl(hidden_states: torch.Tensor,
         global_num_experts = E
     # without an expert map (rejected above) every expert is local
     assert global_num_experts == E, "global_num_experts must equal the number of local experts (no expert parallelism)"
-    # Narrower than the reference's Triton kernel, which masks ragged K and N
-    # (for_moe/fused_moe.py:191-205,218-223): rows are moved in 16-byte chunks.
-    # (16 bytes of the weight dtype: 16 e4m3, 8 bf16 / fp16, 4 fp32 elements)
-    chunk = 16 // w1.element_size()
-    assert hidden_states.size(1) % chunk == 0 and (N // 2) % chunk == 0, \
-        f"hidden size and intermediate size must be multiples of {chunk}"
-    # (the stride of a dimension of size 1 carries no meaning)
-    assert all(t.stride(dim) % chunk == 0 for t in (w1, w2) for dim in (0, 1) if t.size(dim) > 1), \
-        f"weight strides must be multiples of {chunk} elements"
-    assert all(t.data_ptr() % 16 == 0 for t in (hidden_states, w1, w2)), "tensors must be 16-byte aligned"
+    # Like the reference's Triton kernel, which masks ragged K and N
+    # (for_moe/fused_moe.py:191-205,218-223), any hidden and intermediate size is taken with
+    # 16-bit and fp32 weights: rows that are not whole, aligned 16-byte chunks go through an
+    # element-by-element kernel.  e4m3 rows are moved in 16-byte chunks only (the reference has
+    # no such path):
+    if fp8:
+        assert hidden_states.size(1) % 16 == 0 and (N // 2) % 16 == 0, \
+            "hidden size and intermediate size must be multiples of 16 with e4m3 weights"
+        # (the stride of a dimension of size 1 carries no meaning)
+        assert all(t.stride(dim) % 16 == 0 for t in (w1, w2) for dim in (0, 1) if t.size(dim) > 1), \
+            "weight strides must be multiples of 16 elements with e4m3 weights"
+        assert all(t.data_ptr() % 16 == 0 for t in (hidden_states, w1, w2)), "tensors must be 16-byte aligned"
     _lib.require_gpu_tensor(hidden_states, "hidden_states")
     top_k_num = topk_ids.size(1)
     CHUNK_SIZE: int = 64 * 1024

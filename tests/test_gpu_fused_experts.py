@@ -778,3 +778,66 @@ def test_fused_moe_layer_with_tiled_weights(moe, oracle, dev):
     assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
     tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
     _close(outs[1], oracle.fused_experts_ref(x, w13, w2, tw, ids))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("E,H,I,T,K", [(8, 100, 52, 33, 2), (4, 66, 30, 17, 2), (16, 1001, 333, 200, 4),
+                                       (3, 7, 5, 9, 1), (8, 130, 70, 300, 2)])
+def test_ragged_hidden_and_intermediate_sizes(moe, oracle, dev, dtype, E, H, I, T, K):
+    """H and I that are not multiples of 16 bytes: the reference's Triton kernel masks the K tail
+    and the N edge (nanovllm/layers/for_moe/fused_moe.py:191-205,218-223); here both GEMM
+    passes run on the element-by-element variant of the register-staged kernel, which rounds
+    where the reference stores."""
+    print(f"ragged {dtype} E={E} H={H} I={I} T={T} K={K}", flush=True)
+    x, w13, w2, logits = _layer(E, H, I, T, K, 3 + H + T, dtype, wstd=0.05 if H < 500 else 0.02)
+    tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
+    out = moe.fused_experts(x.to(dev), w13.to(dev), w2.to(dev), None, None, tw.to(dev), ids.to(dev))
+    torch.cuda.synchronize()
+    assert out.dtype == dtype and out.shape == x.shape
+    if dtype == torch.float32:
+        _close(out, oracle.fused_experts_ref(x, w13, w2, tw, ids), rtol=1e-4, atol=1e-5)
+    else:
+        _close(out, oracle.fused_experts_ref(x, w13, w2, tw, ids))
+        _close(out, oracle.fused_experts_ref(x, w13, w2, tw, ids, mirror_rounding=True), rtol=1.6e-2, atol=2e-3)
+
+
+@pytest.mark.parametrize("bm", [32, 64, 128, 256])
+def test_ragged_sizes_with_every_block_size_bias_and_activations(moe, oracle, dev, bm, monkeypatch):
+    E, H, I, T, K = 8, 100, 52, 150, 2
+    x, w13, w2, logits = _layer(E, H, I, T, K, 31, torch.bfloat16)
+    g = torch.Generator().manual_seed(4)
+    b13 = (torch.randn(E, 2 * I, generator=g) * 0.1).bfloat16()
+    b2 = (torch.randn(E, H, generator=g) * 0.1).bfloat16()
+    tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
+    monkeypatch.setattr(moe.fused_moe, "try_get_optimal_moe_config", lambda *a, **k: {"BLOCK_SIZE_M": bm})
+    d = lambda t: t.to(dev)
+    for act in ("silu", "swigluoai", "gelu"):
+        print(f"ragged bm={bm} {act}", flush=True)
+        out = moe.fused_experts(d(x), d(w13), d(w2), d(b13), d(b2), d(tw), d(ids), activation=act)
+        _close(out, oracle.fused_experts_ref(x, w13, w2, tw, ids, activation=act, w1_bias=b13, w2_bias=b2,
+                                             mirror_rounding=True), rtol=2e-2, atol=4e-3)
+        _close(out, oracle.fused_experts_ref(x, w13, w2, tw, ids, activation=act, w1_bias=b13, w2_bias=b2))
+
+
+def test_element_aligned_tensors_and_odd_strides_equal_the_aligned_call(moe, dev):
+    """The same numbers behind a base address that is only element-aligned, and behind weight rows
+    with a stride that is not a multiple of 16 bytes: the element-by-element kernel rounds where
+    the tuned kernels of this block size do, so the results are equal bit for bit."""
+    E, H, I, T, K = 8, 128, 64, 70, 2
+    x, w13, w2, logits = _layer(E, H, I, T, K, 77, torch.bfloat16)
+    d = lambda t: t.to(dev)
+    tw, ids, _ = moe.fused_topk(d(x), d(logits), K, True)
+    cfg = {"BLOCK_SIZE_M": 64}   # the register-staged kernel in both calls
+    import unittest.mock as mock
+    with mock.patch.object(moe.fused_moe, "try_get_optimal_moe_config", lambda *a, **k: cfg):
+        want = moe.fused_experts(d(x), d(w13), d(w2), None, None, tw, ids)
+        xs = torch.empty(T * H + 1, dtype=torch.bfloat16, device=dev)[1:].view(T, H)       # base + 2 bytes
+        xs.copy_(x)
+        w13s = torch.empty(E, 2 * I, H + 3, dtype=torch.bfloat16, device=dev)[:, :, :H]     # row stride H + 3
+        w13s.copy_(w13)
+        w2s = torch.empty(E * H * I + 1, dtype=torch.bfloat16, device=dev)[1:].view(E, H, I)
+        w2s.copy_(w2)
+        assert xs.data_ptr() % 16 != 0 and w13s.stride(1) % 8 != 0
+        got = moe.fused_experts(xs, w13s, w2s, None, None, tw, ids)
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))

@@ -138,27 +138,30 @@ def test_fused_experts_shape_assertions(moe):
         moe.fused_experts(x, w1, w2, None, None, tw, ids, activation="relu")
 
 
-def test_fused_experts_states_its_narrower_contract(moe):
-    """The reference's Triton kernel masks ragged K and N (for_moe/fused_moe.py:191-205,218-223);
-    this build moves rows in 16-byte chunks and says so where the reference asserts."""
+def test_fused_experts_takes_ragged_sizes_except_with_e4m3(moe):
+    """The reference's Triton kernel masks ragged K and N (for_moe/fused_moe.py:191-205,218-223).
+    So does this build for 16-bit and fp32 weights (an element-by-element kernel): such calls pass
+    every host check and stop at the device check here.  e4m3 rows move in 16-byte chunks only."""
     tw = torch.zeros(4, 2)
     ids = torch.zeros(4, 2, dtype=torch.int32)
     x = torch.zeros(4, 60, dtype=torch.bfloat16)
-    with pytest.raises(AssertionError, match="multiples of 8"):
+    with pytest.raises(RuntimeError, match="no CPU path"):           # H = 60
         moe.fused_experts(x, torch.zeros(2, 32, 60, dtype=torch.bfloat16), torch.zeros(2, 60, 16, dtype=torch.bfloat16),
                           None, None, tw, ids)
     x = torch.zeros(4, 64, dtype=torch.bfloat16)
-    with pytest.raises(AssertionError, match="multiples of 8"):
+    with pytest.raises(RuntimeError, match="no CPU path"):           # I = 12
         moe.fused_experts(x, torch.zeros(2, 24, 64, dtype=torch.bfloat16), torch.zeros(2, 64, 12, dtype=torch.bfloat16),
                           None, None, tw, ids)
     w1 = torch.zeros(2, 32, 68, dtype=torch.bfloat16)[:, :, :64]      # row stride 68
-    with pytest.raises(AssertionError, match="weight strides"):
-        moe.fused_experts(x, w1, torch.zeros(2, 64, 16, dtype=torch.bfloat16), None, None, tw, ids)
-    # 16 bytes are four fp32 elements: H = 60 passes the size rule in fp32 (and stops at the device check)
     with pytest.raises(RuntimeError, match="no CPU path"):
-        moe.fused_experts(torch.zeros(4, 60), torch.zeros(2, 24, 60), torch.zeros(2, 60, 12), None, None, tw, ids)
-    with pytest.raises(AssertionError, match="multiples of 4"):
+        moe.fused_experts(x, w1, torch.zeros(2, 64, 16, dtype=torch.bfloat16), None, None, tw, ids)
+    with pytest.raises(RuntimeError, match="no CPU path"):           # fp32, H = 62
         moe.fused_experts(torch.zeros(4, 62), torch.zeros(2, 24, 62), torch.zeros(2, 62, 12), None, None, tw, ids)
+    # e4m3: multiples of 16 elements
+    f8 = torch.float8_e4m3fn
+    with pytest.raises(AssertionError, match="multiples of 16"):
+        moe.fused_experts(torch.zeros(4, 72, dtype=torch.bfloat16), torch.zeros(2, 32, 72).to(f8), torch.zeros(2, 72, 16).to(f8),
+                          None, None, tw, ids, per_channel_quant=True, w1_scale=torch.ones(2, 32), w2_scale=torch.ones(2, 72))
     # the stride of a dimension of size 1 says nothing: one expert cut out of a larger tensor
     one13 = torch.zeros(3, 32, 64, dtype=torch.bfloat16).as_strided((1, 32, 64), (2051, 64, 1))
     one2 = torch.zeros(3, 64, 16, dtype=torch.bfloat16)[:1]
