@@ -841,3 +841,40 @@ def test_element_aligned_tensors_and_odd_strides_equal_the_aligned_call(moe, dev
         got = moe.fused_experts(xs, w13s, w2s, None, None, tw, ids)
     torch.cuda.synchronize()
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+def _random_ragged_cases(n, seed):
+    import random
+    rnd = random.Random(seed)
+    cases = []
+    for i in range(n):
+        E = rnd.choice([1, 3, 8, 40])
+        K = rnd.choice([k for k in (1, 2, 4) if k <= E])
+        H, I = rnd.randint(3, 300), rnd.randint(2, 200)
+        if rnd.random() < 0.3:
+            H = 64 * rnd.randint(1, 4)          # only I ragged: the gate-up pass alone would suit the tuned kernels
+        T = rnd.choice([1, 5, 33, 100, 257, 600])
+        bm = rnd.choice([0, 32, 64, 128, 256])
+        cases.append((i, E, K, H, I, T, bm, rnd.choice(["bf16", "f16", "f32"])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_ragged_cases(16, 4711), ids=lambda c: "-".join(map(str, c)))
+def test_random_ragged_shapes(moe, oracle, dev, case, monkeypatch):
+    """Seeded random hidden / intermediate sizes with no regard for 16-byte chunks, every block size
+    and dtype, against the oracle that rounds where the reference stores."""
+    i, E, K, H, I, T, bm, dt = case
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dt]
+    x, w13, w2, logits = _layer(E, H, I, T, K, 2000 + i, dtype)
+    tw, ids, _ = oracle.topk_softmax(logits, K, renormalize=True)
+    if bm:
+        monkeypatch.setattr(moe.fused_moe, "try_get_optimal_moe_config", lambda *a, **k: {"BLOCK_SIZE_M": bm})
+    d = lambda t: t.to(dev)
+    out = moe.fused_experts(d(x), d(w13), d(w2), None, None, d(tw), d(ids))
+    if dtype == torch.float32:
+        _close(out, oracle.fused_experts_ref(x, w13, w2, tw, ids), rtol=1e-4, atol=1e-5)
+    else:
+        ragged = H % 8 != 0 or I % 8 != 0
+        mode = True if ragged else _mode(moe, T, E, K, H, dtype, bm=bm or None)
+        _close(out, oracle.fused_experts_ref(x, w13, w2, tw, ids, mirror_rounding=mode), rtol=1.6e-2,
+               atol=2e-3 + 4e-3 * out.float().abs().max().item())
