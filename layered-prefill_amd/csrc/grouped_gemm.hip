@@ -509,9 +509,10 @@ __device__ __forceinline__ uint32_t pack2<ElemF16>(float a, float b) {
 struct BigCtx {
   const char* a_base;   // wave-uniform base of the A rows
   const char* w_base;   // wave-uniform base of this expert's weights
-  uint32_t a_off[8];    // per-lane byte offsets of the eight 32-row load groups
+  uint32_t a_off[8];    // per-lane byte offsets of the wavefront's eight requests of a unit (dma_win_bias included)
   uint32_t w_off[8];
-  uint32_t dma_lds;     // LDS offset of this wavefront's DMA window in unit slot 0, group 0
+  uint32_t dma_lds;     // LDS address of the middle of this wavefront's 8 KB DMA window in unit slot 0
+  uint32_t dma_lds_light_a;  // the same for the 2 KB window of the first 64-row token unit of a weight-streaming tile
   int rd_k[4];          // fragment read offsets for the four MFMA steps of a K tile
   int x_row;            // byte offset of this wavefront's first token row in a token unit
   int w_row[4];         // byte offsets of this wavefront's weight fragments in a weight unit
@@ -529,18 +530,40 @@ __device__ __forceinline__ void static_for(F&& f) {
   }
 }
 
-// 16 bytes per lane from global memory into LDS at unit_lds + GROUP * 4096 + 16 * lane: the
-// destination offset goes into M0 with one scalar addition, the wait state M0 needs is the s_nop.
-template <int GROUP>
-__device__ __forceinline__ void lds_dma16_group(const char* base, uint32_t lane_byte_offset, uint32_t unit_lds) {
-  asm volatile(
-      "s_add_u32 m0, %0, %3\n\t"
-      "s_nop 0\n\t"
-      "global_load_lds_dwordx4 %1, %2"
-      :
-      : "s"(unit_lds), "v"(lane_byte_offset), "s"(base), "n"(GROUP * 4096)
-      : "memory", "scc");
+// 16 bytes per lane from global memory into LDS, the instruction's offset field added on both
+// sides: the data of base + lane_byte_offset + OFF lands at M0 + OFF + 16 * lane.  A wavefront fills
+// one contiguous window of a unit (8 KB of a 32 KB unit) with requests that differ in OFF only, so
+// M0 is written once per window (SET_M0, on the first request; the s_nop is the wait state M0
+// needs) instead of once per request: three scalar writes and wait states per K tile where there
+// were sixteen (0.5 to 1 % of the launch at 8448 and at 256 tokens, results unchanged bit for bit).
+// M0 has to keep its value from one request of a window to the next; nothing else in the K loops
+// writes it (they are MFMAs, LDS reads, waits and these requests).
+template <int OFF, bool SET_M0>
+__device__ __forceinline__ void lds_dma16_rel(const char* base, uint32_t lane_byte_offset, uint32_t lds_m0) {
+  static_assert(OFF >= -4096 && OFF <= 4095, "13-bit signed offset field");
+  if constexpr (SET_M0) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %1, %2 offset:%3"
+        :
+        : "s"(lds_m0), "v"(lane_byte_offset), "s"(base), "n"(OFF)
+        : "memory");
+  } else {
+    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(lane_byte_offset), "s"(base), "n"(OFF) : "memory");
+  }
 }
+// Request J (0..7) of a wavefront's 8 KB window of a 32 KB unit; lds_mid = LDS address of the
+// window's middle.  Unit byte 8192 * wave + 1024 * J + 16 * lane, i.e. row 64 * wave + 8 * J +
+// lane / 8 of the unit, position lane % 8 of that row.
+template <int J, bool SET_M0>
+__device__ __forceinline__ void lds_dma16_win(const char* base, uint32_t lane_byte_offset, uint32_t lds_mid) {
+  lds_dma16_rel<(J - 4) * 1024, SET_M0>(base, lane_byte_offset, lds_mid);
+}
+// What a per-lane offset of request J carries besides the data's offset from the operand's start:
+// the offset field's share taken out again, and 4096 that the base pointers are short of (so that
+// no offset is negative).
+constexpr uint32_t dma_win_bias(int j) { return static_cast<uint32_t>(4096 - (j - 4) * 1024); }
 
 // Main loop for a wavefront that has FMC live token fragments (0..4).
 // Unit j of the stream  A(0) W(0) A(1) W(1) ...  lives in ring slot j % 5.
@@ -634,8 +657,8 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
     // request q of the tile's first STEPS-1 steps: W(kt+1)[4..7], then A(kt+2)[0..7]
     auto req = [&](auto qt) {
       constexpr int q = decltype(qt)::value;
-      if constexpr (q < 4) { if constexpr (DO_W) lds_dma16_group<4 + q>(w1, c.w_off[4 + q], lds_fa); }
-      else { if constexpr (DO_A) lds_dma16_group<q - 4>(a2, c.a_off[q - 4], lds_fw); }
+      if constexpr (q < 4) { if constexpr (DO_W) lds_dma16_win<4 + q, q == 0>(w1, c.w_off[4 + q], lds_fa); }
+      else { if constexpr (DO_A) lds_dma16_win<q - 4, q == 4>(a2, c.a_off[q - 4], lds_fw); }
     };
     using One = IntTag<1>;
     if constexpr (STEPS == 4) {
@@ -661,7 +684,7 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
     const uint32_t lds_w2 = c.dma_lds + fa;  // W(kt+2) takes the token unit of the tile just finished
     step(IntTag<4>{}, IntTag<NEXT ? 1 : 0>{}, IntTag<0>{}, wfQ, xfQ, wfP, xfP, sa, sw, [&](auto it) {
       constexpr int i = decltype(it)::value;
-      if constexpr (NEXT_W) lds_dma16_group<i>(w2, c.w_off[i], lds_w2);
+      if constexpr (NEXT_W) lds_dma16_win<i, i == 0>(w2, c.w_off[i], lds_w2);
     });
     a2 += c.a_step;
     w1 += c.w_step;
@@ -669,10 +692,14 @@ __device__ __forceinline__ void big_mainloop(const BigCtx& c, const char* smem, 
 
   // fill the ring: W(0) and half of W(1) were requested by the caller as soon as it knew
   // the expert; A(0) and A(1) follow here.  Then wait for tile 0 only.
-  static_for<0, 8>([&](auto it) { lds_dma16_group<decltype(it)::value>(c.a_base, c.a_off[decltype(it)::value], c.dma_lds); });
+  static_for<0, 8>([&](auto it) {
+    constexpr int i = decltype(it)::value;
+    lds_dma16_win<i, i == 0>(c.a_base, c.a_off[i], c.dma_lds);
+  });
   if (1 < nk) {
     static_for<0, 8>([&](auto it) {
-      lds_dma16_group<decltype(it)::value>(c.a_base + c.a_step, c.a_off[decltype(it)::value], c.dma_lds + 2 * kBigUnitBytes);
+      constexpr int i = decltype(it)::value;
+      lds_dma16_win<i, i == 0>(c.a_base + c.a_step, c.a_off[i], c.dma_lds + 2 * kBigUnitBytes);
     });
     wait_vmcnt<kBigDmaPerUnit>();
   } else {
@@ -718,17 +745,26 @@ __device__ __forceinline__ void big_light_mainloop(const BigCtx& c, const char* 
   };
   auto a_slot = [](int k) { return 4 * kBigUnitBytes + (k & 3) * kTokUnit; };
   auto issue_w = [&](int k) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) lds_dma16(c.w_base + k * c.w_step, c.w_off[i], c.dma_lds + w_slot(k) + i * 4096);
+    const char* const src = c.w_base + k * c.w_step;
+    const uint32_t mid = c.dma_lds + w_slot(k);
+    static_for<0, 8>([&](auto it) {
+      constexpr int i = decltype(it)::value;
+      lds_dma16_win<i, i == 0>(src, c.w_off[i], mid);
+    });
   };
+  // a token unit is 64 rows: the wavefront's window is 2 KB, two requests around its middle
   auto issue_a = [&](int k) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) lds_dma16(c.a_base + k * c.a_step, c.a_off[i], c.dma_lds + a_slot(k) + i * 4096);
+    const char* const src = c.a_base + k * c.a_step;
+    const uint32_t mid = c.dma_lds_light_a + (k & 3) * kTokUnit;
+    lds_dma16_rel<-1024, true>(src, c.a_off[0], mid);
+    lds_dma16_rel<0, false>(src, c.a_off[1], mid);
   };
   // request order: W(0) W(1) (first half by the caller) A(0) A(1) W(2) A(2), then W(k) A(k) per K tile
   if (1 < nk) {
-#pragma unroll
-    for (int i = 4; i < 8; ++i) lds_dma16(c.w_base + c.w_step, c.w_off[i], c.dma_lds + w_slot(1) + i * 4096);
+    static_for<4, 8>([&](auto it) {
+      constexpr int i = decltype(it)::value;
+      lds_dma16_win<i, i == 4>(c.w_base + c.w_step, c.w_off[i], c.dma_lds + w_slot(1));
+    });
   }
   issue_a(0);
   if (1 < nk) issue_a(1);
@@ -1032,23 +1068,28 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
   constexpr int ES = Mma::kEs, CH = Mma::kBigChunks;
   const int nk = p.Kd / (kBigRowBytes / ES);
   BigCtx c;
-  const int ld_row = tid >> 3;                        // row inside a 32-row load group
-  const int ld_chunk = (tid & 7) ^ ((tid >> 4) & 7);  // logical chunk this lane fetches
-  c.a_base = static_cast<const char*>(p.a);
-  c.w_base = static_cast<const char*>(p.w) + static_cast<int64_t>(e) * p.w_stride_e * ES;
-  c.dma_lds = __builtin_amdgcn_readfirstlane(lds_offset_of(smem) + wave * 1024);
+  // DMA geometry: wavefront w fills bytes [8192 w, 8192 w + 8192) of every unit with eight requests
+  // of 1 KB; request j of lane l is unit row 64 w + 8 j + l / 8, position l % 8 of that row, which
+  // holds the row's 16-byte chunk (l % 8) ^ ((row >> 1) & 7).  The base pointers are 4096 short of
+  // the operands (dma_win_bias).
+  const int dma_row0 = 64 * wave + (lane >> 3);
+  auto dma_chunk = [&](int row) { return (lane & 7) ^ ((row >> 1) & 7); };
+  c.a_base = static_cast<const char*>(p.a) - 4096;
+  c.w_base = static_cast<const char*>(p.w) + static_cast<int64_t>(e) * p.w_stride_e * ES - 4096;
+  c.dma_lds = __builtin_amdgcn_readfirstlane(lds_offset_of(smem) + wave * 8192 + 4096);
+  c.dma_lds_light_a = __builtin_amdgcn_readfirstlane(lds_offset_of(smem) + 4 * kBigUnitBytes + wave * 2048 + 1024);
   c.a_step = c.w_step = kBigRowBytes;
   if (p.w_tiled) {
-    // unit (n-tile, K tile) of this expert is one 32 KB piece in LDS order: thread tid moves bytes
-    // [16 tid, 16 tid + 16) of each of its eight 4 KB groups
+    // unit (n-tile, K tile) of this expert is one 32 KB piece in LDS order: every request reads
+    // the bytes it writes
     c.w_base += static_cast<int64_t>(nt) * nk * kBigUnitBytes;
     c.w_step = kBigUnitBytes;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) c.w_off[i] = static_cast<uint32_t>(i * 4096 + tid * 16);
+    for (int i = 0; i < 8; ++i) c.w_off[i] = static_cast<uint32_t>(wave * 8192 + i * 1024 + lane * 16) + dma_win_bias(i);
   } else {
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const int rr = ld_row + 32 * i;
+    const int rr = dma_row0 + 8 * i;
     int64_t wrow;
     if constexpr (GATED) {
       const int half = rr >> 7;
@@ -1059,18 +1100,21 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
       const int n = n0 + rr;
       wrow = n < p.N ? n : p.N - 1;
     }
-    c.w_off[i] = static_cast<uint32_t>(wrow * p.w_stride_n * ES + ld_chunk * 16);
+    c.w_off[i] = static_cast<uint32_t>(wrow * p.w_stride_n * ES + dma_chunk(rr) * 16) + dma_win_bias(i);
   }
   }
   // The weights of the first K tile and a half are on their way (ring slots 1 and 3) while
   // the slot ids are still being looked at: they are the cold half of the fill.
   // Neither slot overlaps the side arrays above.
-#pragma unroll
-  for (int i = 0; i < 8; ++i) lds_dma16(c.w_base, c.w_off[i], c.dma_lds + kBigUnitBytes + i * 4096);
+  static_for<0, 8>([&](auto it) {
+    constexpr int i = decltype(it)::value;
+    lds_dma16_win<i, i == 0>(c.w_base, c.w_off[i], c.dma_lds + kBigUnitBytes);
+  });
   if (1 < nk) {  // the first half of W(1); the main loops request the second
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      lds_dma16(c.w_base + c.w_step, c.w_off[i], c.dma_lds + 3 * kBigUnitBytes + i * 4096);
+    static_for<0, 4>([&](auto it) {
+      constexpr int i = decltype(it)::value;
+      lds_dma16_win<i, i == 0>(c.w_base + c.w_step, c.w_off[i], c.dma_lds + 3 * kBigUnitBytes);
+    });
   }
   __syncthreads();
   const int nvalid = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
@@ -1095,28 +1139,34 @@ __device__ __forceinline__ void big_tile(const GemmParams& p, int mb, int nt, ch
     if (p.w_scale) my_ws = p.w_scale[e * p.w_scale_stride_e + wr];
     if (p.bias) my_bias = El::ld(static_cast<const typename El::S*>(p.bias)[e * p.bias_stride_e + wr]);
   }
-  const int a_groups = (nvalid + 31) >> 5;  // 32-row token groups that hold real slots
   if (p.a_tiled) {
     // the block's rows of K tile kt are unit (mb, kt), written in LDS order by the gate-up pass
     c.a_base += static_cast<int64_t>(mb) * nk * kBigUnitBytes;
     c.a_step = kBigUnitBytes;
   }
+  // A weight-streaming tile (at most 64 real slots) loads token units of 64 rows: there the
+  // wavefront's window is 2 KB, rows 16 w + 8 j + l / 8, two requests with the offsets -1024 and 0.
+  const bool light_a = nvalid <= 64;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    // groups made of padding only re-request group 0 (an L1 hit) so that every
-    // token unit is exactly eight loads and the vmcnt bookkeeping stays fixed
-    const int gi = i < a_groups ? i : 0;
+    int row = light_a ? 16 * wave + 8 * (i & 1) + (lane >> 3) : dma_row0 + 8 * i;
+    const uint32_t bias = light_a ? static_cast<uint32_t>(4096 - ((i & 1) - 1) * 1024) : dma_win_bias(i);
+    // a request whose eight rows are all padding asks for rows 0..7 again (an L1 hit), so that
+    // every token unit is the same number of loads and the vmcnt bookkeeping stays fixed
+    const bool dead = (row & ~7) >= nvalid;
+    const int pos_row = row;   // the row whose place in LDS the data takes (it decides the chunk order)
+    if (dead) row = lane >> 3;
     if (p.a_tiled) {
-      c.a_off[i] = static_cast<uint32_t>(gi * 4096 + tid * 16);
+      // (a dead request reads the bytes of live rows 0..7 into its own place: never looked at)
+      c.a_off[i] = static_cast<uint32_t>(row * kBigRowBytes + (lane & 7) * 16) + bias;
       continue;
     }
-    const int slot = mb * kBigBM + ld_row + 32 * gi;
-    int64_t src = slot;
+    int64_t src = static_cast<int64_t>(mb) * kBigBM + row;
     if (!p.a_by_slot) {
-      const int tok = s_tok[ld_row + 32 * gi];
+      const int tok = s_tok[row];
       src = tok < p.numel ? tok / p.top_k : 0;
     }
-    c.a_off[i] = static_cast<uint32_t>(src * p.lda * ES + ld_chunk * 16);
+    c.a_off[i] = static_cast<uint32_t>(src * p.lda * ES + dma_chunk(pos_row) * 16) + bias;
   }
   // chunk ch of MFMA step kk: lane half lhi owns the K elements of chunks CH * (2 kk + lhi) .. + CH - 1
 #pragma unroll
@@ -1659,7 +1709,9 @@ int launch(const GemmParams& p, hipStream_t s) {
 static bool dma_offsets_fit(const GemmParams& p, bool gated, int64_t sorted_cap, int es) {
   const int64_t a_rows = p.a_by_slot ? sorted_cap : p.numel / p.top_k;
   const int64_t w_rows = gated ? 2LL * p.N : p.N;
-  return a_rows * p.lda * es < (1LL << 32) && w_rows * p.w_stride_n * es < (1LL << 32);
+  // (16 KB of head room: the per-lane offsets carry up to 8 KB on top of the data's offset)
+  const int64_t limit = (1LL << 32) - 16384;
+  return a_rows * p.lda * es < limit && w_rows * p.w_stride_n * es < limit;
 }
 
 // Whether a 16-bit pass runs on the large-tile kernel.
